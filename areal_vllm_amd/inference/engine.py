@@ -30,10 +30,11 @@ import torch
 from ..api.cli_args import InferenceServerConfig
 from ..models import hf_io
 from ..models.config import ModelConfig
+from ..models import build_model
 from ..models.transformer import Transformer
 from ..ops.attention import PAGE_SIZE
 from ..utils import logging
-from .model_runner import ModelRunner
+from .model_runner import HybridModelRunner, ModelRunner
 
 logger = logging.getLogger("inference-engine")
 
@@ -64,7 +65,7 @@ def _kv_bytes_per_page(cfg: ModelConfig, n_layers: int, hkv: int, elt: int = 2) 
 class NativeInferenceEngine:
     def __init__(self, config: InferenceServerConfig, model_config: Optional[ModelConfig] = None,
                  device: Optional[torch.device] = None, tp_size: int = 1, tp_rank: int = 0, tp_group=None,
-                 num_pages: Optional[int] = None, kv_cache_gb: Optional[float] = None):
+                 num_pages: Optional[int] = None, kv_cache_gb: Optional[float] = None, score_mode: bool = False):
         if _runtime is None:
             raise RuntimeError(f"C++ runtime extension missing ({_runtime_err}); run `python build_ext.py`")
         self.config = config
@@ -77,6 +78,9 @@ class NativeInferenceEngine:
         self.tp_size, self.tp_rank, self.tp_group = tp_size, tp_rank, tp_group
         self._num_pages_arg = num_pages
         self._kv_cache_gb = kv_cache_gb
+        # scoring (`replay_step`): decode plans keep the fp32 logits of their step, logits are computed in fp32
+        self.score_mode = bool(score_mode)
+        self._replays: Dict[str, list] = {}  # request id -> [scheduler id, tokens fed so far]
         self.model: Optional[Transformer] = None
         self.runner: Optional[ModelRunner] = None
         self.sched = None
@@ -127,8 +131,9 @@ class NativeInferenceEngine:
     def initialize(self, load_weights: bool = True):
         cfg, mc = self.config, self.model_config
         cfg.reject_unsupported()
-        self.model = Transformer(mc, dtype=self.dtype, device=self.device, tp_size=self.tp_size, tp_rank=self.tp_rank,
+        self.model = build_model(mc, dtype=self.dtype, device=self.device, tp_size=self.tp_size, tp_rank=self.tp_rank,
                                  tp_group=self.tp_group)
+        hybrid = bool(getattr(self.model, "hybrid", False))
         self.model.requires_grad_(False)
         self.model.eval()
         self.model.flatten()
@@ -144,9 +149,15 @@ class NativeInferenceEngine:
         else:
             self.model.init_weights(seed=1)
         ctx = int(cfg.context_length or mc.max_position_embeddings)
-        hkv = self.model.layers[0].attn.hkv
         kv_fp8 = str(cfg.kv_cache_dtype) in ("fp8", "fp8_e4m3")
-        per_page = _kv_bytes_per_page(mc, len(self.model.layers), hkv, 1 if kv_fp8 else 2)
+        if hybrid:
+            assert not kv_fp8, "layer-list decoders keep their caches in the model's dtype"
+            elt = torch.empty((), dtype=self.dtype).element_size()
+            per_page = max(1, sum(g * (d + v) for g, d, v in (blk.mix.cache_shape() for blk in self.model.layers
+                                                             if blk.kind == "attention")) * PAGE_SIZE * elt)
+        else:
+            hkv = self.model.layers[0].attn.hkv
+            per_page = _kv_bytes_per_page(mc, len(self.model.layers), hkv, 1 if kv_fp8 else 2)
         if self._num_pages_arg is not None:
             num_pages = int(self._num_pages_arg)
         elif self._kv_cache_gb is not None:
@@ -160,9 +171,18 @@ class NativeInferenceEngine:
         num_pages = max(8, num_pages)
         max_running = int(cfg.max_running_requests or 256)
         self.decode_steps = max(1, int(cfg.num_continuous_decode_steps))
-        self.runner = ModelRunner(self.model, num_pages, ctx, max_running, decode_steps=self.decode_steps,
-                                  use_graph=not cfg.disable_cuda_graph, seed=int(cfg.random_seed),
-                                  buckets=cfg.cuda_graph_bs, kv_dtype=torch.float8_e4m3fn if kv_fp8 else None)
+        # models with recurrent layers: one state slot per request the scheduler may hold
+        recurrent = hybrid and bool(getattr(mc, "has_recurrent_state", False))
+        if hybrid:
+            self.runner = HybridModelRunner(self.model, num_pages, ctx, max_running,
+                                            n_state_slots=max_running if recurrent else 0,
+                                            decode_steps=self.decode_steps, use_graph=not cfg.disable_cuda_graph,
+                                            seed=int(cfg.random_seed), buckets=cfg.cuda_graph_bs)
+        else:
+            self.runner = ModelRunner(self.model, num_pages, ctx, max_running, decode_steps=self.decode_steps,
+                                      use_graph=not cfg.disable_cuda_graph, seed=int(cfg.random_seed),
+                                      buckets=cfg.cuda_graph_bs, kv_dtype=torch.float8_e4m3fn if kv_fp8 else None)
+        self.runner.keep_logits = self.score_mode
         self.num_pages = num_pages
         self.runner.tune_decode_paths()
         if (self.tp_size > 1 and self.device.type == "cuda" and not cfg.disable_custom_all_reduce
@@ -188,7 +208,10 @@ class NativeInferenceEngine:
         sc.max_prefill_tokens = int(cfg.max_prefill_tokens)
         sc.context_length = ctx
         sc.decode_steps = self.decode_steps
-        sc.enable_prefix_cache = not cfg.disable_radix_cache
+        # a cached prefix holds keys and values, not the recurrent state its tokens left behind
+        sc.enable_prefix_cache = not cfg.disable_radix_cache and not recurrent
+        sc.num_state_slots = max_running if recurrent else 0
+        sc.paged_prefill = hybrid
         sc.policy = cfg.schedule_policy if cfg.schedule_policy in ("fcfs", "lpm") else "fcfs"
         sc.schedule_conservativeness = float(cfg.schedule_conservativeness)
         self.sched = _runtime.Scheduler(sc)
@@ -512,6 +535,77 @@ class NativeInferenceEngine:
         if prompts:
             ev.wait()
         return out  # type: ignore
+
+    # ------------------------------------------------------------------------ scoring of given tokens
+    def open_replay(self, rid: str):
+        """Admit a request whose tokens the caller supplies step by step (`replay_step`); nothing is sampled."""
+        assert self.tp_size == 1, "replay requests are served by one rank"
+
+        def f():
+            if rid in self._replays:
+                raise ValueError(f"duplicate request id {rid}")
+            sid = self.sched.open_replay(rid)
+            if sid < 0:
+                raise RuntimeError("every recurrent-state slot is in use")
+            self._replays[rid] = [sid, 0]
+        self._control(f)
+
+    def close_replay(self, rid: str):
+        """The request is over: its pages and its state slot are free again."""
+        def f():
+            ent = self._replays.pop(rid, None)
+            if ent is not None:
+                self.sched.close_replay(ent[0])
+        self._control(f)
+
+    def replay_step(self, entries: List[Any]) -> np.ndarray:
+        """One engine step over given tokens. `entries`: (request id, next tokens, places among them whose logits
+        are wanted). Portions of several tokens, and first tokens, form one prefill plan; single tokens of requests
+        that have context form one decode plan (the decode graph's kernels) - the two plans of a step are issued back
+        to back. Returns the wanted logits, fp32 [n, vocab], in the order of the entries and their places. Needs an
+        engine made with `score_mode`."""
+        assert self.score_mode, "replay_step needs an engine constructed with score_mode=True"
+
+        def f():
+            self._finish_inflight()
+            pre, dec = [], []
+            for k, (rid, toks, want) in enumerate(entries):
+                ent = self._replays[rid]
+                single = len(toks) == 1 and ent[1] > 0 and self.decode_steps == 1
+                (dec if single else pre).append((k, ent, [int(t) for t in toks], [int(w) for w in want]))
+            got: Dict[int, torch.Tensor] = {}
+            if pre:
+                plan = self.sched.plan_replay([e[1][0] for e in pre], [e[2] for e in pre], False)
+                if plan["kind"] != 1:
+                    raise RuntimeError("the page pool cannot hold this step's tokens")
+                cu = plan["cu_q"]
+                rows = [int(cu[i]) + w for i, e in enumerate(pre) for w in e[3]]
+                plan["logit_rows"] = np.asarray(rows, dtype=np.int64)
+                self.runner.kept_logits = None
+                self.runner.prefill(plan)
+                self.sched.process_replay(plan["plan_id"])
+                self.stats["prefill_steps"] += 1
+                at = 0
+                for i, e in enumerate(pre):
+                    got[e[0]] = self.runner.kept_logits[at:at + len(e[3])]
+                    at += len(e[3])
+            if dec:
+                plan = self.sched.plan_replay([e[1][0] for e in dec], [e[2] for e in dec], True)
+                if plan["kind"] != 2:
+                    raise RuntimeError("the page pool cannot hold this step's tokens")
+                self.runner.decode(plan)
+                self.sched.process_replay(plan["plan_id"])
+                self.stats["decode_steps"] += 1
+                logits = self.runner.static[self.runner._last_decode[0]]["logits"]
+                for i, e in enumerate(dec):
+                    got[e[0]] = logits[i:i + 1] if e[3] else logits[:0]
+            for _, ent, toks, _ in pre + dec:
+                ent[1] += len(toks)
+            outs = [got[k] for k in range(len(entries)) if got[k].shape[0]]
+            if not outs:
+                return np.zeros((0, self.model_config.vocab_size), np.float32)
+            return torch.cat(outs, 0).float().cpu().numpy()
+        return self._control(f)
 
     # ------------------------------------------------------------------------ control API
     def pause(self):
@@ -911,6 +1005,8 @@ def assign_hf_named_tensors(model: Transformer, tensors: Dict[str, torch.Tensor]
     tensor whose name maps onto no parameter of this model raises instead of being dropped (a silent drop
     leaves that part of the rollout model on stale weights)."""
     cfg = model.cfg
+    if getattr(model, "hybrid", False):
+        return model.assign_named_tensors(tensors, strict)
     if cfg.family == "gpt2":
         return _assign_gpt2_named_tensors(model, tensors, strict)
     D = cfg.head_dim

@@ -55,19 +55,9 @@ class ModelRunner:
         if not self.buckets or self.buckets[-1] < max_batch:
             self.buckets.append(max_batch)
         cfg = self.cfg
-        self.hq = model.layers[0].attn.hq
-        self.hkv = model.layers[0].attn.hkv
-        # kv_dtype: torch.float8_e4m3fn stores the cache as e4m3 bytes (None: the model's dtype)
-        self.kv = [ops.alloc_kv_cache(num_pages, self.hkv, cfg.head_dim, kv_dtype or self.dtype, self.device)
-                   for _ in model.layers]
-        if cfg.pos_embed == "rope":
-            self.rope = model.rope(self.device)
-        else:
-            # learned absolute positions (GPT-2) are added to the embeddings; q and k go into attention and the
-            # cache unrotated: the rotate-and-write kernels run on a table of angle zero
-            self.rope = ops.RotaryTable(cfg.head_dim, 1, device=self.device)
-            self.rope.cos.fill_(1.0)
-            self.rope.sin.zero_()
+        self.keep_logits = False  # decode plans leave the fp32 logits of their last step in the static buffers
+        self.kept_logits: Optional[torch.Tensor] = None  # prefill plans with `logit_rows`: logits at those rows
+        self._alloc_caches(kv_dtype)
         # LayerNorm with bias, projections with bias, the MLP without a gate (GPT-2): the unfused layer body
         self.plain_family = cfg.norm_type != "rms" or not cfg.mlp_gated or cfg.linear_bias or cfg.pos_embed != "rope"
         self.step_counter = torch.zeros(1, dtype=torch.int64, device=self.device)
@@ -109,6 +99,22 @@ class ModelRunner:
         # qkv projection with bias + RoPE + KV-cache write in its epilogue (head sizes that are multiples of 64)
         self.fused_qkv_rope = (cfg.head_dim % 64 == 0 and not cfg.qk_norm
                                and os.environ.get("AREAL_FUSED_QKV_ROPE", "1") != "0")
+
+    def _alloc_caches(self, kv_dtype):
+        cfg, model = self.cfg, self.model
+        self.hq = model.layers[0].attn.hq
+        self.hkv = model.layers[0].attn.hkv
+        # kv_dtype: torch.float8_e4m3fn stores the cache as e4m3 bytes (None: the model's dtype)
+        self.kv = [ops.alloc_kv_cache(self.num_pages, self.hkv, cfg.head_dim, kv_dtype or self.dtype, self.device)
+                   for _ in model.layers]
+        if cfg.pos_embed == "rope":
+            self.rope = model.rope(self.device)
+        else:
+            # learned absolute positions (GPT-2) are added to the embeddings; q and k go into attention and the
+            # cache unrotated: the rotate-and-write kernels run on a table of angle zero
+            self.rope = ops.RotaryTable(cfg.head_dim, 1, device=self.device)
+            self.rope.cos.fill_(1.0)
+            self.rope.sin.zero_()
 
     # ------------------------------------------------------------------- vision-language requests
     def _placeholder_mask(self, prompt_ids: List[int], grid_thw: torch.Tensor):
@@ -272,7 +278,7 @@ class ModelRunner:
             dist.broadcast(tok, src=src, group=self.model.tp_group)
             dist.broadcast(lp, src=src, group=self.model.tp_group)
 
-    def _final_logits(self, h, residual) -> torch.Tensor:
+    def _final_logits(self, h, residual, fp32: bool = False) -> torch.Tensor:
         cfg = self.cfg
         if cfg.norm_type != "rms":
             from ..models.transformer import add_norm
@@ -280,6 +286,8 @@ class ModelRunner:
             x, _ = add_norm(cfg, h, self.model.norm, getattr(self.model, "norm_bias", None), residual)
         else:
             x, _ = ops.rmsnorm(h, self.model.norm, cfg.rms_norm_eps, residual, cfg.gemma_norm)
+        if fp32:
+            return F.linear(x.float(), self.model.head_weight.float())
         return F.linear(x, self.model.head_weight)
 
     # ----------------------------------------------------------------------------- prefill
@@ -296,10 +304,9 @@ class ModelRunner:
         max_q = int(plan["max_q"])
         B = len(plan["req_ids"])
         T = ids.numel()
-        hq, hkv, D = self.hq, self.hkv, self.cfg.head_dim
         self.n_prefill_tokens += T
 
-        rope = self.rope
+        rope = getattr(self, "rope", None)
         if self.is_vl and any(int(r) in self.mm for r in plan["req_ids"].tolist()):
             h, pos3 = self._multimodal_prefill_inputs(plan, ids)
             rope = self.model.mrope(pos3)  # per-token table, addressed by the token's index in the plan
@@ -308,23 +315,15 @@ class ModelRunner:
             h = self.model.embed_tokens(ids, pos)
         if self.cfg.pos_embed != "rope":
             pos = torch.zeros_like(pos)  # the only row of the angle-zero table
-        residual = None
-        for li, blk in enumerate(self.model.layers):
-            kc, vc = self.kv[li]
-
-            def attn_fn(blk_, qkv2d, kc=kc, vc=vc):
-                qkv = qkv2d.view(T, hq + 2 * hkv, D)
-                ops.rope_and_cache_write_(qkv, pos, slots, rope, kc, vc, hq, hkv)
-                q = qkv[:, :hq]
-                if has_prefix:  # some row has context in the cache: attention reads the pages directly
-                    out = ops.flash_attn_paged_prefill(q, kc, vc, bt, cu_q, cu_k, max_q)
-                else:
-                    out, _ = ops.flash_attn_varlen(q, qkv[:, hq:hq + hkv], qkv[:, hq + hkv:], cu_q, cu_q, max_q)
-                return out
-
-            h, residual = self._layer(blk, h, residual, pos, slots, attn_fn)
+        h, residual = self._prefill_layers(plan, h, pos, slots, rope, cu_q, cu_k, bt, max_q)
+        if plan.get("logit_rows") is not None:  # scoring: fp32 logits at chosen tokens of the packed batch
+            rows = torch.from_numpy(np.asarray(plan["logit_rows"], dtype=np.int64)).to(dev)
+            self.kept_logits = self._final_logits(h[rows], None if residual is None else residual[rows],
+                                                  fp32=True).float()
+            if not np.any(plan["sample"]):  # nothing to draw: a plan that only scores
+                return np.zeros(B, np.int64), np.zeros(B, np.float32)
         last = (cu_q[1:] - 1).long()
-        logits = self._final_logits(h[last], residual[last])
+        logits = self._final_logits(h[last], None if residual is None else residual[last])
         temp = torch.from_numpy(plan["temperature"]).to(dev)
         top_p = torch.from_numpy(plan["top_p"]).to(dev)
         top_k = torch.from_numpy(np.minimum(plan["top_k"], self.V).astype(np.int32)).to(dev)
@@ -341,6 +340,28 @@ class ModelRunner:
         if self.ipc_ar is not None:
             self.ipc_ar.raise_if_error()
         return tok_h, lp_h
+
+    def _prefill_layers(self, plan, h, pos, slots, rope, cu_q, cu_k, bt, max_q):
+        """All layers of a packed prefill batch -> (last sublayer output, residual stream)."""
+        hq, hkv, D = self.hq, self.hkv, self.cfg.head_dim
+        T = h.shape[0]
+        has_prefix = bt is not None
+        residual = None
+        for li, blk in enumerate(self.model.layers):
+            kc, vc = self.kv[li]
+
+            def attn_fn(blk_, qkv2d, kc=kc, vc=vc):
+                qkv = qkv2d.view(T, hq + 2 * hkv, D)
+                ops.rope_and_cache_write_(qkv, pos, slots, rope, kc, vc, hq, hkv)
+                q = qkv[:, :hq]
+                if has_prefix:  # some row has context in the cache: attention reads the pages directly
+                    out = ops.flash_attn_paged_prefill(q, kc, vc, bt, cu_q, cu_k, max_q)
+                else:
+                    out, _ = ops.flash_attn_varlen(q, qkv[:, hq:hq + hkv], qkv[:, hq + hkv:], cu_q, cu_q, max_q)
+                return out
+
+            h, residual = self._layer(blk, h, residual, pos, slots, attn_fn)
+        return h, residual
 
     # ------------------------------------------------------------------ penalty count table
     def token_counts(self) -> "ops.TokenCounts":
@@ -369,7 +390,7 @@ class ModelRunner:
     def _alloc_static(self, Bp: int) -> Dict[str, torch.Tensor]:
         dev = self.device
         k = self.decode_steps
-        nsplit = ops.decode_num_splits(Bp, self.hkv, 4096, fp8=ops.attention.is_fp8(self.kv[0][0]))
+        nsplit, ws = self._decode_workspace(Bp)
         st = dict(
             input_ids=torch.zeros(Bp, dtype=torch.int64, device=dev),
             positions=torch.zeros(Bp, dtype=torch.int32, device=dev),
@@ -392,14 +413,17 @@ class ModelRunner:
             penalty_slot=torch.full((Bp,), -1, dtype=torch.int32, device=dev),
             freq_pen=torch.zeros(Bp, dtype=torch.float32, device=dev),
             pres_pen=torch.zeros(Bp, dtype=torch.float32, device=dev),
+            state_slots=torch.full((Bp,), -1, dtype=torch.int32, device=dev),
         )
         st["nsplit"] = nsplit
-        st["ws"] = ops.DecodeWorkspace(Bp, self.hq, self.cfg.head_dim, nsplit, dev) if nsplit > 1 else None
+        st["ws"] = ws
+        if self.keep_logits:
+            st["logits"] = torch.zeros(Bp, self.V, dtype=torch.float32, device=dev)
         # Pinned host memory, two sets used alternately: uploads of plan n+1 are written while the copies of
         # plan n may still be queued, and plan n's results are read while plan n+1 fills the other set.
         if dev.type == "cuda":
             st["host"] = [dict(i64=torch.zeros(2, Bp, dtype=torch.int64).pin_memory(),
-                               i32=torch.zeros(8, Bp, dtype=torch.int32).pin_memory(),
+                               i32=torch.zeros(9, Bp, dtype=torch.int32).pin_memory(),
                                f32=torch.zeros(4, Bp, dtype=torch.float32).pin_memory(),
                                stop=torch.zeros(Bp, self.n_stop_ids, dtype=torch.int32).pin_memory(),
                                bt=torch.zeros(Bp, self.max_pages, dtype=torch.int32).pin_memory(),
@@ -408,6 +432,11 @@ class ModelRunner:
                                ar_err=torch.zeros(1, dtype=torch.int32).pin_memory(),
                                done=torch.cuda.Event()) for _ in range(2)]
         return st
+
+    def _decode_workspace(self, Bp: int):
+        """(key-range splits, split workspace) of the decode attention at this batch bucket."""
+        nsplit = ops.decode_num_splits(Bp, self.hkv, 4096, fp8=ops.attention.is_fp8(self.kv[0][0]))
+        return nsplit, (ops.DecodeWorkspace(Bp, self.hq, self.cfg.head_dim, nsplit, self.device) if nsplit > 1 else None)
 
     FUSED_MIN_BATCH = 1  # the hand-written layer wins at every batch size (1.8 against 3.5 ms per step at one row)
 
@@ -559,9 +588,7 @@ class ModelRunner:
 
     def _decode_body(self, st: Dict[str, torch.Tensor], filtered: bool, penalized: bool = False):
         """`decode_steps` decode iterations on the static buffers (captured into a graph)."""
-        hq, hkv, D = self.hq, self.hkv, self.cfg.head_dim
         Bp = st["input_ids"].numel()
-        qkv_stride = (hq + 2 * hkv) * D
         fused = self.fused_decode and Bp >= self.FUSED_MIN_BATCH
         pen = {}
         if penalized:
@@ -572,7 +599,6 @@ class ModelRunner:
                           st["block_tables"])
         for s in range(self.decode_steps):
             h = self.model.embed_tokens(st["input_ids"], st["positions"])
-            residual = None
             rope_pos = st["positions"] if self.cfg.pos_embed == "rope" else st["zero_pos"]
             if self.is_vl:  # generated tokens of a request with images sit `delta` away from their index
                 torch.add(st["positions"], st["rope_delta"], out=st["rope_pos"])
@@ -580,18 +606,9 @@ class ModelRunner:
             if fused:
                 logits = self._lm_head(self._decode_layers_fused(st, h, rope_pos))
             else:
-                for li, blk in enumerate(self.model.layers):
-                    kc, vc = self.kv[li]
-
-                    def attn_fn(blk_, qkv2d, kc=kc, vc=vc, rope_pos=rope_pos):
-                        qkv = qkv2d.view(Bp, hq + 2 * hkv, D)
-                        ops.rope_and_cache_write_(qkv, rope_pos, st["slots"], self.rope, kc, vc, hq, hkv)
-                        return ops.paged_attention_decode(qkv[:, :hq], kc, vc, st["block_tables"], st["context_lens"],
-                                                          nsplit=st["nsplit"], workspace=st["ws"],
-                                                          q_row_stride=qkv_stride)
-
-                    h, residual = self._layer(blk, h, residual, st["positions"], st["slots"], attn_fn)
-                logits = self._final_logits(h, residual)
+                logits = self._decode_step_logits(st, h, rope_pos)
+            if self.keep_logits:
+                st["logits"].copy_(logits)
             ops.sample(logits, st["temperature"], st["top_k"] if filtered else None, st["top_p"] if filtered else None,
                        self.seed, self.step_counter, bump_step=True, out_tokens=st["out_tokens"][s],
                        out_logprobs=st["out_logprobs"][s], active=st["active"], **pen)
@@ -599,6 +616,25 @@ class ModelRunner:
             ops.decode_advance_(st["out_tokens"][s], st["input_ids"], st["positions"], st["context_lens"],
                                 st["slots"], st["block_tables"], st["active"], st["remaining"], st["min_remaining"],
                                 st["stop_ids"])
+
+    def _decode_step_logits(self, st, h, rope_pos) -> torch.Tensor:
+        """One decode step of all layers on the unfused path: embeddings [Bp, H] -> logits."""
+        hq, hkv, D = self.hq, self.hkv, self.cfg.head_dim
+        Bp = h.shape[0]
+        qkv_stride = (hq + 2 * hkv) * D
+        residual = None
+        for li, blk in enumerate(self.model.layers):
+            kc, vc = self.kv[li]
+
+            def attn_fn(blk_, qkv2d, kc=kc, vc=vc, rope_pos=rope_pos):
+                qkv = qkv2d.view(Bp, hq + 2 * hkv, D)
+                ops.rope_and_cache_write_(qkv, rope_pos, st["slots"], self.rope, kc, vc, hq, hkv)
+                return ops.paged_attention_decode(qkv[:, :hq], kc, vc, st["block_tables"], st["context_lens"],
+                                                  nsplit=st["nsplit"], workspace=st["ws"],
+                                                  q_row_stride=qkv_stride)
+
+            h, residual = self._layer(blk, h, residual, st["positions"], st["slots"], attn_fn)
+        return self._final_logits(h, residual)
 
     _STATE_KEYS = ("input_ids", "positions", "context_lens", "slots", "active", "remaining", "min_remaining")
 
@@ -711,7 +747,7 @@ class ModelRunner:
                 hi64, hf32, hstop = host["i64"], host["f32"], host["stop"]
                 hi64.zero_()
                 hi32[:4].zero_(); hi32[5:].zero_()
-                hi32[1].fill_(1); hi32[2].fill_(self.V); hi32[5].fill_(1); hi32[7].fill_(-1)
+                hi32[1].fill_(1); hi32[2].fill_(self.V); hi32[5].fill_(1); hi32[7].fill_(-1); hi32[8].fill_(-1)
                 hf32[0].fill_(1.0); hf32[1].fill_(1.0); hf32[2].zero_(); hf32[3].zero_()
                 hstop.fill_(-1)
                 hi64[0, :B] = torch.from_numpy(plan["input_ids"].astype(np.int64))
@@ -725,6 +761,8 @@ class ModelRunner:
                 hi32[5, :B] = torch.from_numpy(plan["remaining"])
                 hi32[6, :B] = torch.from_numpy(plan["min_remaining"])
                 hi32[7, :B] = torch.from_numpy(plan["penalty_slot"])
+                if len(plan.get("state_slots", ())) == B:
+                    hi32[8, :B] = torch.from_numpy(plan["state_slots"])
                 hf32[0, :B] = torch.from_numpy(plan["temperature"])
                 hf32[1, :B] = torch.from_numpy(plan["top_p"])
                 hf32[2, :B] = torch.from_numpy(plan["frequency_penalty"])
@@ -732,7 +770,8 @@ class ModelRunner:
                 hstop[:B] = torch.from_numpy(plan["stop_ids"])
                 for name, src in (("input_ids", hi64[0]), ("slots", hi64[1]), ("positions", hi32[0]),
                                   ("context_lens", hi32[1]), ("top_k", hi32[2]), ("remaining", hi32[5]),
-                                  ("min_remaining", hi32[6]), ("penalty_slot", hi32[7]), ("temperature", hf32[0]),
+                                  ("min_remaining", hi32[6]), ("penalty_slot", hi32[7]), ("state_slots", hi32[8]),
+                                  ("temperature", hf32[0]),
                                   ("top_p", hf32[1]), ("freq_pen", hf32[2]), ("pres_pen", hf32[3]), ("stop_ids", hstop)):
                     st[name].copy_(src, non_blocking=True)
                 st["active"].fill_(1)  # decode_begin retires the padded rows through `kill`
@@ -742,6 +781,8 @@ class ModelRunner:
                                         ("context_lens", plan["context_lens"], 1), ("top_k", top_k, self.V),
                                         ("remaining", plan["remaining"], 1), ("min_remaining", plan["min_remaining"], 0),
                                         ("penalty_slot", plan["penalty_slot"], -1),
+                                        ("state_slots", plan["state_slots"] if len(plan.get("state_slots", ())) == B
+                                         else np.full(B, -1, np.int32), -1),
                                         ("temperature", plan["temperature"], 1.0), ("top_p", plan["top_p"], 1.0),
                                         ("freq_pen", plan["frequency_penalty"], 0.0),
                                         ("pres_pen", plan["presence_penalty"], 0.0)):
@@ -795,3 +836,112 @@ class ModelRunner:
 
     def kv_cache_bytes(self) -> int:
         return sum(k.numel() * k.element_size() + v.numel() * v.element_size() for k, v in self.kv)
+
+
+class HybridModelRunner(ModelRunner):
+    """Runner of layer-list decoders (``models/hybrid.py``): the same plans, graphs, sampler and bookkeeping as
+    ``ModelRunner``; per layer a paged window cache (attention mixers; key and value sizes from the layer) or a set
+    of fp32 state slots (recurrent mixers), an fp32 residual stream normalised after every sum.
+
+    Prompt portions and decoded tokens run the same kernels: attention reads keys and values from the pages only
+    (the portion's own tokens are written first), so a position's result does not depend on how its prompt was cut;
+    the recurrence continues from the row's state slot, or from zero when the row's first token has position 0."""
+
+    def __init__(self, model, num_pages: int, max_context: int, max_batch: int, n_state_slots: int = 0, **kw):
+        self.n_state_slots = max(1, int(n_state_slots))
+        kw["fused_decode"] = False
+        super().__init__(model, num_pages, max_context, max_batch, **kw)
+        self.fused_decode = False
+        self.plain_family = True
+
+    def _alloc_caches(self, kv_dtype):
+        from ..ops import mlstm as mlstm_ops
+        from ..ops import window_attention as wattn
+
+        assert kv_dtype is None, "layer-list decoders keep their caches in the model's dtype"
+        self.hq = self.hkv = 1
+        self.kv, self.state = [], []
+        for blk in self.model.layers:
+            if blk.kind == "attention":
+                G, D, V = blk.mix.cache_shape()
+                self.kv.append(wattn.alloc_window_cache(self.num_pages, G, D, V, self.dtype, self.device))
+                self.state.append(None)
+            else:
+                H, D, V = blk.mix.state_shape()
+                self.kv.append(None)
+                self.state.append(mlstm_ops.RecurrentState(self.n_state_slots, H, D, V, self.device))
+        self._neg1 = torch.full((1,), -1, dtype=torch.int32, device=self.device)
+
+    def kv_cache_bytes(self) -> int:
+        return (sum(k.numel() * k.element_size() + v.numel() * v.element_size() for k, v in filter(None, self.kv))
+                + sum(s.nbytes() for s in self.state if s is not None))
+
+    # ------------------------------------------------------------------------------ layers
+    def _run_layers(self, xc: torch.Tensor, st) -> torch.Tensor:
+        """Embeddings (compute dtype) -> fp32 residual stream after the last layer."""
+        from ..ops.post_norm import scaled_add_norm
+
+        cfg = self.cfg
+        x32 = xc.float() if xc.dtype != torch.float32 else xc.clone()
+        alpha, eps = float(cfg.postln_alpha), float(cfg.rms_norm_eps)
+        trace = getattr(self, "layer_trace", None)
+        for li, blk in enumerate(self.model.layers):
+            y = blk.mix.step(xc, st, self.kv[li] if blk.kind == "attention" else self.state[li])
+            x32, xc = scaled_add_norm(x32, y, blk.norm1, alpha, eps, self.dtype)
+            if blk.norm2 is not None:
+                y = blk.mlp(xc) if blk.mlp is not None else None
+                x32, xc = scaled_add_norm(x32, y, blk.norm2, alpha, eps, self.dtype)
+            if trace is not None:
+                trace.append(x32.clone())
+        return x32
+
+    def _final_logits(self, h, residual, fp32: bool = False) -> torch.Tensor:
+        from ..ops.post_norm import scaled_add_norm
+
+        x32, xc = scaled_add_norm(h.contiguous(), None, self.model.norm, 1.0, float(self.cfg.rms_norm_eps),
+                                  self.dtype, inplace=False)
+        if fp32 or self.keep_logits:
+            return F.linear(x32, self.model.head_weight.float())
+        return F.linear(xc, self.model.head_weight)
+
+    def _prefill_layers(self, plan, h, pos, slots, rope, cu_q, cu_k, bt, max_q):
+        from ..models.hybrid import StepTensors
+
+        dev = self.device
+        assert bt is not None, "layer-list decoders read their context from the pages: the plan needs page tables"
+        B = len(plan["req_ids"])
+        first = plan["positions"][plan["cu_q"][:-1]].astype(np.int32)
+        ss = plan.get("state_slots")
+        ss = np.asarray(ss, dtype=np.int32) if ss is not None and len(ss) == B else np.full(B, -1, np.int32)
+        if any(s is not None for s in self.state):
+            assert (ss >= 0).all() and (ss < self.n_state_slots).all(), "a row of the plan has no state slot"
+        st = StepTensors(cu_q, torch.from_numpy(plan["chunk_end"].astype(np.int32)).to(dev), max_q, slots, bt,
+                         torch.from_numpy(first).to(dev), torch.from_numpy(ss).to(dev))
+        return self._run_layers(h, st), None
+
+    # ------------------------------------------------------------------------------ decode
+    def _decode_workspace(self, Bp: int):
+        from ..ops import window_attention as wattn
+
+        nsplit, ws = 1, None
+        mixers = [blk.mix for blk in self.model.layers if blk.kind == "attention"]
+        if mixers and self.device.type == "cuda":
+            nsplit = max(wattn.decode_splits(Bp, m.shape.window, self.max_context) for m in mixers)
+            if nsplit > 1:
+                hv = max(m.H * m.V for m in mixers)
+                hh = max(m.H for m in mixers)
+                ws = (torch.empty(Bp * nsplit * hv, dtype=torch.float32, device=self.device),
+                      torch.empty(Bp * nsplit * hh * 2, dtype=torch.float32, device=self.device))
+        return nsplit, ws
+
+    def _decode_step_logits(self, st, h, rope_pos) -> torch.Tensor:
+        from ..models.hybrid import StepTensors
+
+        Bp = h.shape[0]
+        if "cu_rows" not in st:
+            st["cu_rows"] = torch.arange(Bp + 1, dtype=torch.int32, device=self.device)
+        # rows that are retired (no cache slot) touch no state slot either
+        eff = torch.where(st["slots"] < 0, self._neg1, st["state_slots"])
+        step = StepTensors(st["cu_rows"], st["context_lens"], 1, st["slots"], st["block_tables"], st["positions"], eff,
+                           nsplit=st["nsplit"], workspace=st["ws"])
+        return self._final_logits(self._run_layers(h, step), None)

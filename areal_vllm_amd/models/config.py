@@ -12,6 +12,10 @@ import os
 from typing import Any, Dict, List, Optional
 
 
+# config.json "architecture" -> reader in models/hybrid.py (designs given as a list of layers)
+LAYER_LIST_DESIGNS = {"Kuzanex": "kuzanex_config"}
+
+
 @dataclasses.dataclass
 class ModelConfig:
     family: str = "qwen2"
@@ -118,6 +122,10 @@ class ModelConfig:
     # ------------------------------------------------------------------ HF interop
     @classmethod
     def from_hf_dict(cls, d: Dict[str, Any], is_critic: bool = False) -> "ModelConfig":
+        if d.get("architecture") in LAYER_LIST_DESIGNS:  # layer-list decoders describe themselves layer by layer
+            from . import hybrid
+
+            return getattr(hybrid, LAYER_LIST_DESIGNS[d["architecture"]])(d)
         if d.get("model_type") in ("qwen2_vl", "qwen2_5_vl") and "text_config" in d:
             # nested layout: language model settings under text_config, tower under vision_config
             text = dict(d["text_config"])
@@ -191,7 +199,12 @@ class ModelConfig:
     @classmethod
     def from_pretrained(cls, path: str, is_critic: bool = False) -> "ModelConfig":
         with open(os.path.join(path, "config.json")) as f:
-            return cls.from_hf_dict(json.load(f), is_critic=is_critic)
+            d = json.load(f)
+        if d.get("architecture") in LAYER_LIST_DESIGNS:
+            from . import hybrid
+
+            return getattr(hybrid, LAYER_LIST_DESIGNS[d["architecture"]] + "_from_dir")(path)
+        return cls.from_hf_dict(d, is_critic=is_critic)
 
     def to_hf_dict(self) -> Dict[str, Any]:
         if self.vision is not None:

@@ -137,6 +137,8 @@ def _gather_vocab(model, t: torch.Tensor, group) -> torch.Tensor:
 
 def load_hf_weights(model, path: str, strict: bool = True) -> None:
     """Fill `model` (a ``Transformer``, possibly a TP shard / pipeline stage) from a HF checkpoint."""
+    if getattr(model, "hybrid", False):  # layer-list decoders keep their checkpoint's own tensor names
+        return model.load_checkpoint(path, strict=strict)
     cfg: ModelConfig = model.cfg
     rd = _ShardReader(path)
     tp, tr = model.tp_size, model.tp_rank

@@ -1,0 +1,140 @@
+"""Sliding-window attention over the paged cache with shaped scores: soft cap, linear distance bias, mixing of the
+heads' scores ahead of the softmax, an optional value-less sink in the denominator.
+
+GPU: ``csrc/hip/window_attn.hip`` (one kernel for prompt portions and, with a split key range, for decoding).
+CPU: a PyTorch formulation used by the unit tests and CPU runs.
+
+Cache layout: K [pages, G, 32, D], V [pages, G, 32, Dv] (token-major pages; key and value sizes may differ).
+"""
+import dataclasses
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib as L
+from .attention import PAGE_SIZE
+
+
+@dataclasses.dataclass
+class ScoreShape:
+    """Constants of the score pipeline (see the module docstring)."""
+    scale: float
+    softcap: float = 0.0  # <= 0: no cap
+    slope_exp: float = 0.0  # slope of head h: 2^(-slope_exp (h + 1) / H); 0: no distance bias
+    window: int = 0  # <= 0: all earlier tokens
+    sink: bool = False
+
+
+def alloc_window_cache(num_pages: int, n_kv_heads: int, k_dim: int, v_dim: int, dtype, device
+                       ) -> Tuple[torch.Tensor, torch.Tensor]:
+    return (torch.zeros(num_pages, n_kv_heads, PAGE_SIZE, k_dim, dtype=dtype, device=device),
+            torch.zeros(num_pages, n_kv_heads, PAGE_SIZE, v_dim, dtype=dtype, device=device))
+
+
+def qk_norm_cache_write(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                        slots: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, n_heads: int, eps: float
+                        ) -> torch.Tensor:
+    """proj [T, >= (H + G) D + G Dv]: q heads | k heads | v heads (more columns may follow). RMS-normalises every q
+    and k head over D (times the weight vector, shared by the heads), writes k and v of tokens with slot >= 0 into the
+    paged caches and returns the normalised queries [T, H, D]."""
+    T = proj.shape[0]
+    G, D, V = kcache.shape[1], kcache.shape[3], vcache.shape[3]
+    H = n_heads
+    assert proj.stride(1) == 1 and proj.shape[1] >= (H + G) * D + G * V
+    q = torch.empty(T, H, D, dtype=proj.dtype, device=proj.device)
+    if L.use_hip(proj):
+        assert slots.dtype == torch.int64 and kcache.dtype == proj.dtype
+        L.check(L.lib().areal_qk_norm_cache_write(
+            L.ptr(proj), L.c_int64(proj.stride(0)), L.ptr(q_weight), L.ptr(k_weight), L.ptr(slots), L.ptr(q),
+            L.ptr(kcache), L.ptr(vcache), L.c_int(T), L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_float(eps),
+            L.c_int(L.dtype_flag(proj)), L.stream_ptr()), "qk_norm_cache_write")
+        return q
+    qk = proj[:, :(H + G) * D].float().view(T, H + G, D)
+    qk = qk * torch.rsqrt(qk.pow(2).mean(-1, keepdim=True) + eps)
+    qn, kn = qk[:, :H], qk[:, H:]
+    if q_weight is not None:
+        qn = qn * q_weight.float()
+    if k_weight is not None:
+        kn = kn * k_weight.float()
+    q.copy_(qn)
+    ok = slots >= 0
+    if ok.any():
+        pg, off = (slots[ok] // PAGE_SIZE).long(), (slots[ok] % PAGE_SIZE).long()
+        kcache[pg, :, off, :] = kn[ok].to(kcache.dtype)
+        vcache[pg, :, off, :] = proj[ok, (H + G) * D:(H + G) * D + G * V].view(-1, G, V).to(vcache.dtype)
+    return q
+
+
+def decode_splits(batch: int, window: int, max_context: int) -> int:
+    """Key-range splits of a decode launch: enough workgroups to occupy the device, at least a few pages each."""
+    span = max_context if window <= 0 else min(window + PAGE_SIZE, max_context)
+    pages = max(1, (span + PAGE_SIZE - 1) // PAGE_SIZE)
+    return int(max(1, min(256 // max(1, batch), pages // 4, 32)))
+
+
+def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_tables: torch.Tensor,
+                     cu_q: torch.Tensor, ctx_len: torch.Tensor, max_q: int, shape: ScoreShape,
+                     mix: Optional[torch.Tensor] = None, nsplit: int = 1,
+                     workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+    """q [T, H, D] (row b owns tokens cu_q[b]:cu_q[b+1], the LAST positions of its context of ctx_len[b] tokens,
+    whose keys / values are in the cache already). mix [H, H] or None. Returns [T, H, Dv]."""
+    T, H, D = q.shape
+    G, V = kcache.shape[1], vcache.shape[3]
+    B = cu_q.numel() - 1
+    if L.use_hip(q):
+        assert q.is_contiguous() and kcache.dtype == q.dtype and block_tables.dtype == torch.int32
+        assert cu_q.dtype == torch.int32 and ctx_len.dtype == torch.int32 and block_tables.is_contiguous()
+        assert mix is None or (mix.dtype == q.dtype and mix.is_contiguous() and mix.shape == (H, H))
+        out = torch.empty(T, H, V, dtype=q.dtype, device=q.device)
+        want = 1 if max_q == 1 else 16
+        while want > 1 and want // 2 >= max_q:
+            want //= 2
+        bq = int(L.lib().areal_window_attn_tile(L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_int(want)))
+        if bq <= 0:
+            raise RuntimeError(f"window attention: {H} heads of size {D} / {V} do not fit the kernel's tile memory")
+        pa = pm = None
+        if nsplit > 1:
+            assert max_q == 1, "split key ranges are for single-query rows"
+            if workspace is None:
+                workspace = (torch.empty(T, nsplit, H, V, dtype=torch.float32, device=q.device),
+                             torch.empty(T, nsplit, H, 2, dtype=torch.float32, device=q.device))
+            pa, pm = workspace
+            assert pa.numel() >= T * nsplit * H * V and pm.numel() >= T * nsplit * H * 2
+        L.check(L.lib().areal_window_attn(
+            L.ptr(q), L.ptr(kcache), L.ptr(vcache), L.ptr(block_tables), L.c_int(block_tables.shape[1]), L.ptr(cu_q),
+            L.ptr(ctx_len), L.ptr(mix), L.ptr(out), L.ptr(pa), L.ptr(pm), L.c_int(B), L.c_int(int(max_q)), L.c_int(T),
+            L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_int(bq), L.c_float(shape.scale),
+            L.c_float(shape.softcap), L.c_float(shape.slope_exp), L.c_int(int(shape.window)), L.c_int(int(shape.sink)),
+            L.c_int(int(nsplit)), L.c_int(L.dtype_flag(q)), L.stream_ptr()), "window_attn")
+        return out
+    out = torch.zeros(T, H, V, dtype=torch.float32, device=q.device)
+    cq, cl = cu_q.tolist(), ctx_len.tolist()
+    rep = H // G
+    slopes = (torch.tensor([2.0 ** (-shape.slope_exp * (h + 1) / H) for h in range(H)], device=q.device)
+              if shape.slope_exp != 0 else torch.zeros(H, device=q.device))
+    for b in range(B):
+        n, ctx = cq[b + 1] - cq[b], cl[b]
+        if n == 0:
+            continue
+        lo = 0 if shape.window <= 0 else max(0, ctx - n - shape.window + 1)
+        pages = block_tables[b, :(ctx + PAGE_SIZE - 1) // PAGE_SIZE].long()
+        kk = kcache[pages].permute(1, 0, 2, 3).reshape(G, -1, D)[:, lo:ctx].float().repeat_interleave(rep, 0)
+        vv = vcache[pages].permute(1, 0, 2, 3).reshape(G, -1, V)[:, lo:ctx].float().repeat_interleave(rep, 0)
+        s = torch.einsum("ihd,hjd->hij", q[cq[b]:cq[b + 1]].float(), kk) * shape.scale
+        if shape.softcap > 0:
+            s = shape.softcap * torch.tanh(s / shape.softcap)
+        i = torch.arange(ctx - n, ctx, device=q.device).view(n, 1)
+        j = torch.arange(lo, ctx, device=q.device).view(1, -1)
+        s = s - slopes.view(H, 1, 1) * (i - j).float()
+        if mix is not None:
+            s = torch.einsum("hg,gij->hij", mix.float(), s)
+        ok = (i - j >= 0) & ((i - j < shape.window) if shape.window > 0 else True)
+        s = s.masked_fill(~ok, float("-inf"))
+        m = s.max(-1, keepdim=True).values
+        if shape.sink:
+            m = m.clamp(min=0.0)
+        e = torch.exp(s - m)
+        den = e.sum(-1, keepdim=True) + (torch.exp(-m) if shape.sink else 0.0)
+        out[cq[b]:cq[b + 1]] = torch.einsum("hij,hjv->ihv", e / den, vv)
+    return out.to(q.dtype)

@@ -22,6 +22,8 @@ OUT_DIR = ROOT / "areal_vllm_amd" / "_C"
 BUILD_DIR = ROOT / "build"
 ARCH = os.environ.get("AREAL_HIP_ARCH", "gfx950")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# fp32 arithmetic is issued one lane-value at a time: the compiler does not pair it into packed fp32 instructions
+NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 def _newer(src: Path, dst: Path, extra=()) -> bool:
@@ -39,18 +41,21 @@ def _run(cmd):
     return r
 
 
-def build_hip(verbose=True) -> Path:
+def build_hip(verbose=True, only=None) -> Path:
+    """`only`: stems of the sources to build the library from (a program that needs a few kernels of a fresh
+    checkout); the next full build relinks it from everything."""
     BUILD_DIR.mkdir(exist_ok=True)
     OUT_DIR.mkdir(exist_ok=True)
     headers = list(HIP_DIR.glob("*.hpp"))
-    srcs = sorted(HIP_DIR.glob("*.hip"))
+    srcs = sorted(s for s in HIP_DIR.glob("*.hip") if only is None or s.stem in only)
     objs = []
     jobs = []
     for s in srcs:
         o = BUILD_DIR / (s.stem + ".o")
         objs.append(o)
         if _newer(s, o, headers):
-            jobs.append([HIPCC, f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", "-c", str(s), "-o", str(o)])
+            jobs.append([HIPCC, f"--offload-arch={ARCH}", "-O3", "-fPIC", "-std=c++17", *NO_PACKED_FP32, "-c", str(s), "-o",
+                         str(o)])
     if jobs:
         if verbose:
             print(f"[build_ext] compiling {len(jobs)} HIP source(s) for {ARCH}")

@@ -1,0 +1,217 @@
+// Matrix-memory recurrence (mLSTM of the xLSTM family) with a carried, stabilised fp32 state.
+//
+// Per head, with log gates i_t, f_t (fp32), keys / queries of size D and values of size V:
+//
+//   m_t = max(f_t + m_{t-1}, i_t)                      a_t = exp(f_t + m_{t-1} - m_t),  b_t = exp(i_t - m_t)
+//   S_t = a_t S_{t-1} + b_t k_t v_t^T   [D, V]         n_t = a_t n_{t-1} + b_t k_t   [D]
+//   y_t = S_t^T (q_t / sqrt(D)) / (max(|n_t . q_t / sqrt(D)|, exp(-m_t)) + 1e-6)
+//
+// State slots [slots, heads, ...] live in device memory between steps: a row whose first token has position 0
+// starts from S = 0, n = 0, m = 0 whatever its slot held before; a row with a negative slot is skipped.
+//
+// `mlstm_gates`: i = cap tanh((W_i x + b_i) / cap), f = logsigmoid(cap tanh((W_f x + b_f) / cap)) with fp32
+// accumulation of the dot products (the gates enter exponentials of running sums, so they never pass through bf16).
+// `mlstm_scan`: one wave per (row, head, 64 value columns). Lane c keeps column c of S in registers (D values),
+// the wave keeps n spread over its lanes; keys and queries of a few tokens at a time are staged in LDS as fp32. It
+// writes the unnormalised read-out S_t^T q_t, n_t . q_t and m_t; `mlstm_out` divides, applies the per-head RMS norm,
+// the weight and the sigmoid output gate.
+#include "common.hpp"
+
+namespace {
+
+template <typename T> DEVINL float ldf(const T* p, size_t i);
+template <> DEVINL float ldf<bf16_t>(const bf16_t* p, size_t i) { return bf2f(p[i]); }
+template <> DEVINL float ldf<float>(const float* p, size_t i) { return p[i]; }
+template <typename T> DEVINL void stf(T* p, size_t i, float v);
+template <> DEVINL void stf<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f2bf(v); }
+template <> DEVINL void stf<float>(float* p, size_t i, float v) { p[i] = v; }
+
+// w [2 * NH, W]: rows of the input gate's heads, then of the forget gate's; b [2 * NH]
+template <typename T>
+__global__ void __launch_bounds__(256) mlstm_gates_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                           const T* __restrict__ bias, float* __restrict__ ig,
+                                                           float* __restrict__ fg, int W, int NH, float cap) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* xr = x + (size_t)t * W;
+  for (int u = wave; u < 2 * NH; u += 4) {
+    const T* wr = w + (size_t)u * W;
+    float s = 0.f;
+    for (int i = lane; i < W; i += 64) s += ldf<T>(xr, i) * ldf<T>(wr, i);
+    s = wave_sum(s);
+    if (lane == 0) {
+      float z = s + (bias ? ldf<T>(bias, u) : 0.f);
+      if (cap > 0.f) z = cap * tanhf(z / cap);
+      if (u < NH) ig[(size_t)t * NH + u] = z;
+      else fg[(size_t)t * NH + (u - NH)] = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));  // log sigmoid
+    }
+  }
+}
+
+constexpr int TC = 8;  // tokens staged per round
+
+template <typename T, int DP>
+__global__ void __launch_bounds__(64) mlstm_scan_kernel(
+    const T* __restrict__ proj, int64_t row_stride, int q_off, int k_off, int v_off, const float* __restrict__ ig,
+    const float* __restrict__ fg, const int* __restrict__ cu_q, const int* __restrict__ first_pos,
+    const int* __restrict__ state_slots, float* __restrict__ S, float* __restrict__ N, float* __restrict__ M,
+    float* __restrict__ hbuf, float* __restrict__ nq, float* __restrict__ mt, int NH, int D, int V) {
+  constexpr int NN = (DP + 63) / 64;
+  __shared__ float kq[TC][2][DP];
+  const int b = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x;
+  const int col = blockIdx.z * 64 + lane;
+  const bool has = col < V;
+  const int slot = state_slots[b];
+  const int t_lo = cu_q[b], t_hi = cu_q[b + 1];
+  if (slot < 0 || t_hi <= t_lo) return;
+  const bool fresh = first_pos[b] == 0;
+  const size_t sbase = ((size_t)slot * NH + hd) * D;
+  float s[DP], nn[NN];
+#pragma unroll
+  for (int d = 0; d < DP; ++d) s[d] = (!fresh && has && d < D) ? S[(sbase + d) * V + col] : 0.f;
+#pragma unroll
+  for (int i = 0; i < NN; ++i) {
+    const int d = lane + 64 * i;
+    nn[i] = (!fresh && d < D) ? N[sbase + d] : 0.f;
+  }
+  float m = fresh ? 0.f : M[(size_t)slot * NH + hd];
+  const float qscale = 1.f / sqrtf((float)D);
+  for (int tb = t_lo; tb < t_hi; tb += TC) {
+    const int nt = min(TC, t_hi - tb);
+    __syncthreads();
+    for (int i = lane; i < nt * DP; i += 64) {
+      const int d = i % DP, tt = i / DP;
+      const T* row = proj + (size_t)(tb + tt) * row_stride;
+      kq[tt][0][d] = d < D ? ldf<T>(row, k_off + hd * D + d) : 0.f;
+      kq[tt][1][d] = d < D ? ldf<T>(row, q_off + hd * D + d) * qscale : 0.f;
+    }
+    float vv[TC];
+#pragma unroll
+    for (int tt = 0; tt < TC; ++tt)
+      vv[tt] = (tt < nt && has) ? ldf<T>(proj + (size_t)(tb + tt) * row_stride, v_off + hd * V + col) : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < TC; ++tt) {
+      if (tt < nt) {
+        const size_t th = (size_t)(tb + tt) * NH + hd;
+        const float f = fg[th], ii = ig[th];
+        const float m2 = fmaxf(f + m, ii);
+        const float a = expf(f + m - m2), bb = expf(ii - m2);
+        m = m2;
+        const float bv = bb * vv[tt];
+        float hacc = 0.f;
+#pragma unroll
+        for (int d = 0; d < DP; ++d) {
+          s[d] = a * s[d] + bv * kq[tt][0][d];
+          hacc += s[d] * kq[tt][1][d];
+        }
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < NN; ++i) {
+          const int d = lane + 64 * i;
+          if (d < DP) {
+            nn[i] = a * nn[i] + bb * kq[tt][0][d];
+            part += nn[i] * kq[tt][1][d];
+          }
+        }
+        part = wave_sum(part);
+        if (has) hbuf[th * V + col] = hacc;
+        if (blockIdx.z == 0 && lane == 0) {
+          nq[th] = part;
+          mt[th] = m;
+        }
+      }
+    }
+  }
+  if (has) {
+#pragma unroll
+    for (int d = 0; d < DP; ++d)
+      if (d < D) S[(sbase + d) * V + col] = s[d];
+  }
+  if (blockIdx.z == 0) {
+#pragma unroll
+    for (int i = 0; i < NN; ++i) {
+      const int d = lane + 64 * i;
+      if (d < D) N[sbase + d] = nn[i];
+    }
+    if (lane == 0) M[(size_t)slot * NH + hd] = m;
+  }
+}
+
+// y = h / (max(|nq|, exp(-m)) + 1e-6); per head: y / rms(y) * w * sigmoid(gate)
+template <typename T>
+__global__ void __launch_bounds__(256) mlstm_out_kernel(const float* __restrict__ hbuf, const float* __restrict__ nq,
+                                                         const float* __restrict__ mt, const T* __restrict__ gate,
+                                                         int64_t gate_stride, const T* __restrict__ w,
+                                                         T* __restrict__ out, int NH, int V, float eps) {
+  const size_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int hd = wave; hd < NH; hd += 4) {
+    const size_t th = t * NH + hd;
+    const float den = fmaxf(fabsf(nq[th]), expf(-mt[th])) + 1e-6f;
+    float ss = 0.f;
+    for (int v = lane; v < V; v += 64) {
+      const float y = hbuf[th * V + v] / den;
+      ss += y * y;
+    }
+    ss = wave_sum(ss);
+    const float r = 1.f / sqrtf(ss / (float)V + eps);
+    for (int v = lane; v < V; v += 64) {
+      const float y = hbuf[th * V + v] / den * r;
+      const float g = ldf<T>(gate, t * gate_stride + hd * V + v);
+      stf<T>(out, th * V + v, y * ldf<T>(w, hd * V + v) / (1.f + expf(-g)));
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int areal_mlstm_gates(const void* x, const void* w, const void* bias, float* ig, float* fg, int T, int W,
+                                 int NH, float cap, int dt, hipStream_t st) {
+  if (T == 0) return 0;
+  if (dt == 0)
+    hipLaunchKernelGGL(mlstm_gates_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)w,
+                       (const bf16_t*)bias, ig, fg, W, NH, cap);
+  else
+    hipLaunchKernelGGL(mlstm_gates_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)x, (const float*)w,
+                       (const float*)bias, ig, fg, W, NH, cap);
+  return (int)hipGetLastError();
+}
+
+// proj rows hold (at q_off / k_off / v_off) NH query heads of D, NH key heads of D, NH value heads of V.
+// S [slots, NH, D, V], N [slots, NH, D], M [slots, NH] fp32; hbuf [T, NH, V], nq / mt [T, NH] fp32.
+extern "C" int areal_mlstm_scan(const void* proj, int64_t row_stride, int q_off, int k_off, int v_off,
+                                const float* ig, const float* fg, const int* cu_q, const int* first_pos,
+                                const int* state_slots, float* S, float* N, float* M, float* hbuf, float* nq,
+                                float* mt, int B, int NH, int D, int V, int dt, hipStream_t st) {
+  if (B == 0) return 0;
+  if (D > 256 || D <= 0 || V <= 0) return -1;
+  const dim3 grid(B, NH, (V + 63) / 64);
+#define LAUNCH(TT, DPV)                                                                                          \
+  hipLaunchKernelGGL((mlstm_scan_kernel<TT, DPV>), grid, dim3(64), 0, st, (const TT*)proj, row_stride, q_off,    \
+                     k_off, v_off, ig, fg, cu_q, first_pos, state_slots, S, N, M, hbuf, nq, mt, NH, D, V)
+#define PICK(TT)                 \
+  do {                           \
+    if (D <= 32) LAUNCH(TT, 32); \
+    else if (D <= 64) LAUNCH(TT, 64); \
+    else if (D <= 128) LAUNCH(TT, 128); \
+    else LAUNCH(TT, 256);        \
+  } while (0)
+  if (dt == 0) PICK(bf16_t);
+  else PICK(float);
+#undef PICK
+#undef LAUNCH
+  return (int)hipGetLastError();
+}
+
+extern "C" int areal_mlstm_out(const float* hbuf, const float* nq, const float* mt, const void* gate,
+                               int64_t gate_stride, const void* w, void* out, int T, int NH, int V, float eps, int dt,
+                               hipStream_t st) {
+  if (T == 0) return 0;
+  if (dt == 0)
+    hipLaunchKernelGGL(mlstm_out_kernel<bf16_t>, dim3(T), dim3(256), 0, st, hbuf, nq, mt, (const bf16_t*)gate,
+                       gate_stride, (const bf16_t*)w, (bf16_t*)out, NH, V, eps);
+  else
+    hipLaunchKernelGGL(mlstm_out_kernel<float>, dim3(T), dim3(256), 0, st, hbuf, nq, mt, (const float*)gate,
+                       gate_stride, (const float*)w, (float*)out, NH, V, eps);
+  return (int)hipGetLastError();
+}

@@ -1,0 +1,300 @@
+// Causal sliding-window attention over the paged cache whose scores are shaped before the softmax:
+//
+//   s_g(i, j)  = (q_g(i) . k_c(g)(j)) * scale                      c(g) = g / (H / G): grouped key/value heads
+//   s_g       <- cap * tanh(s_g / cap)                             (cap > 0; otherwise left as it is)
+//   s_g       <- s_g - slope_g * (i - j),  slope_g = 2^(-slope_exp * (g + 1) / H)     (slope_exp = 0: no bias)
+//   t_h        = sum_g M[h, g] s_g                                 head mixing (M = null: t_h = s_h)
+//   visible:     0 <= i - j < window                               (window <= 0: every earlier key)
+//   p_h(j)     = exp(t_h(j)) / (sink + sum_j' exp(t_h(j')))        sink = 1: a key of score 0 that has no value
+//   o_h(i)     = sum_j p_h(j) v_c(h)(j)
+//
+// Scores, weights and the accumulation run in fp32 whatever the storage type T (bf16 / fp32) of q, the caches
+// and the output. Because the heads are mixed before the softmax, one workgroup owns ALL heads of a tile of BQ
+// queries: per 32-key page it forms the H raw score tiles in LDS, mixes them, updates the running maximum /
+// denominator of every (head, query) row and accumulates p.v into LDS-resident fp32 accumulators.
+//
+// The same kernel serves prompt portions (tiles of BQ queries, grid x = tiles, y = rows of the batch) and
+// decoding (BQ = 1, grid z = splits of the visible key range whose partial results `window_attn_combine` merges).
+// Queries of row b are the LAST cu_q[b+1] - cu_q[b] positions of its context of ctx_len[b] tokens.
+//
+// Cache layout: K [pages, G, 32, D], V [pages, G, 32, Dv], token-major inside a page.
+#include "common.hpp"
+
+namespace {
+
+constexpr int PAGE = 32;
+
+template <typename T> DEVINL float ldf(const T* p, size_t i);
+template <> DEVINL float ldf<bf16_t>(const bf16_t* p, size_t i) { return bf2f(p[i]); }
+template <> DEVINL float ldf<float>(const float* p, size_t i) { return p[i]; }
+template <typename T> DEVINL void stf(T* p, size_t i, float v);
+template <> DEVINL void stf<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f2bf(v); }
+template <> DEVINL void stf<float>(float* p, size_t i, float v) { p[i] = v; }
+
+// Per token: RMS norm of every query head (-> q_out) and key head (-> K cache) over its D elements with a weight
+// vector shared by the heads, values copied into the V cache. `proj` rows hold q heads | k heads | v heads (and may
+// be longer: row_stride). slots[t] = page * 32 + offset, negative: nothing is cached for this token.
+template <typename T>
+__global__ void __launch_bounds__(256) qk_norm_cache_write_kernel(
+    const T* __restrict__ proj, int64_t row_stride, const T* __restrict__ qw, const T* __restrict__ kw,
+    const int64_t* __restrict__ slots, T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache, int H,
+    int G, int D, int V, float eps) {
+  const int t = blockIdx.x;
+  const T* row = proj + (size_t)t * row_stride;
+  const int64_t slot = slots[t];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t page = slot >= 0 ? (size_t)(slot / PAGE) : 0;
+  const int off = slot >= 0 ? (int)(slot % PAGE) : 0;
+  for (int u = wave; u < H + G; u += 4) {
+    const T* src = row + (size_t)u * D;
+    float ss = 0.f;
+    for (int d = lane; d < D; d += 64) {
+      const float x = ldf<T>(src, d);
+      ss += x * x;
+    }
+    ss = wave_sum(ss);
+    const float r = 1.f / sqrtf(ss / (float)D + eps);
+    if (u < H) {
+      T* dst = q_out + ((size_t)t * H + u) * D;
+      for (int d = lane; d < D; d += 64) stf<T>(dst, d, ldf<T>(src, d) * r * (qw ? ldf<T>(qw, d) : 1.f));
+    } else if (slot >= 0) {
+      T* dst = kcache + ((page * G + (u - H)) * PAGE + off) * D;
+      for (int d = lane; d < D; d += 64) stf<T>(dst, d, ldf<T>(src, d) * r * (kw ? ldf<T>(kw, d) : 1.f));
+    }
+  }
+  if (slot >= 0) {
+    const T* vsrc = row + (size_t)(H + G) * D;
+    for (int i = threadIdx.x; i < G * V; i += 256) {
+      const int c = i / V, v = i % V;
+      vcache[((page * G + c) * PAGE + off) * V + v] = vsrc[i];
+    }
+  }
+}
+
+struct AttnShape {
+  int H, G, D, V, BQ;
+  // LDS layout in floats
+  DEVINL int rows() const { return H * BQ; }
+  __host__ __device__ size_t floats() const {
+    return (size_t)H * BQ * D + (size_t)H * BQ * V + 2 * (size_t)H * BQ * PAGE + (size_t)PAGE * (D + 1) +
+           (size_t)PAGE * V + 3 * (size_t)H * BQ + (size_t)H * H;
+  }
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) window_attn_kernel(
+    const T* __restrict__ q, const T* __restrict__ kcache, const T* __restrict__ vcache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_len, const T* __restrict__ mix, T* __restrict__ out, float* __restrict__ part_acc,
+    float* __restrict__ part_ml, AttnShape sh, float scale, float softcap, float slope_exp, int window, int sink,
+    int nsplit) {
+  extern __shared__ float lds[];
+  const int H = sh.H, G = sh.G, D = sh.D, V = sh.V, BQ = sh.BQ;
+  const int b = blockIdx.y, split = blockIdx.z, tid = threadIdx.x;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
+  const int t0 = blockIdx.x * BQ;
+  if (t0 >= qlen) return;
+  const int nq = min(BQ, qlen - t0);
+  const int ctx = ctx_len[b];
+  const int pos0 = ctx - qlen + t0;  // position of the tile's first query
+  const int R = H * BQ, rep = H / G;
+  float* qs = lds;                       // [H][BQ][D]
+  float* acc = qs + (size_t)R * D;       // [H][BQ][V]
+  float* S1 = acc + (size_t)R * V;       // [H][BQ][32] shaped scores per head
+  float* S2 = S1 + (size_t)R * PAGE;     // [H][BQ][32] mixed scores, then weights
+  float* Kt = S2 + (size_t)R * PAGE;     // [32][D + 1]
+  float* Vt = Kt + PAGE * (D + 1);       // [32][V]
+  float* mrow = Vt + PAGE * V;           // [R] running maximum
+  float* lrow = mrow + R;                // [R] running denominator
+  float* corr = lrow + R;                // [R] rescale factor of the page in flight
+  float* mixs = corr + R;                // [H][H]
+
+  for (int i = tid; i < R * D; i += 256) {
+    const int d = i % D, r = i / D, qi = r % BQ, g = r / BQ;
+    qs[i] = qi < nq ? ldf<T>(q, ((size_t)(q0 + t0 + qi) * H + g) * D + d) : 0.f;
+  }
+  for (int i = tid; i < R * V; i += 256) acc[i] = 0.f;
+  const bool with_sink = sink && split == 0;
+  for (int i = tid; i < R; i += 256) {
+    mrow[i] = with_sink ? 0.f : -1e30f;
+    lrow[i] = with_sink ? 1.f : 0.f;
+  }
+  if (mix)
+    for (int i = tid; i < H * H; i += 256) mixs[i] = ldf<T>(mix, i);
+
+  // visible keys of the tile: [j_lo, j_hi); pages [p_lo, p_hi), this split's share of them
+  const int j_hi = pos0 + nq;
+  const int j_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int p_lo = j_lo / PAGE, p_hi = (j_hi + PAGE - 1) / PAGE;
+  const int per = (p_hi - p_lo + nsplit - 1) / nsplit;
+  const int my_lo = p_lo + split * per, my_hi = min(p_hi, my_lo + per);
+  const float log2e_unused = 0.f;
+  (void)log2e_unused;
+
+  for (int pg = my_lo; pg < my_hi; ++pg) {
+    const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
+    const int jb = pg * PAGE;
+    // ---- shaped scores of every head
+    for (int c = 0; c < G; ++c) {
+      __syncthreads();  // Kt free (and, first time round, the tile set-up visible)
+      const T* kp = kcache + ((page * G + c) * PAGE) * D;
+      for (int i = tid; i < PAGE * D; i += 256) Kt[(i / D) * (D + 1) + i % D] = ldf<T>(kp, i);
+      __syncthreads();
+      for (int e = tid; e < rep * BQ * PAGE; e += 256) {
+        const int kj = e % PAGE, r = e / PAGE, qi = r % BQ, g = c * rep + r / BQ;
+        const float* qv = qs + ((size_t)g * BQ + qi) * D;
+        const float* kv = Kt + kj * (D + 1);
+        float s = 0.f;
+        for (int d = 0; d < D; ++d) s += qv[d] * kv[d];
+        s *= scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        if (slope_exp != 0.f) s -= exp2f(-slope_exp * (float)(g + 1) / (float)H) * (float)(pos0 + qi - (jb + kj));
+        S1[((size_t)g * BQ + qi) * PAGE + kj] = s;
+      }
+    }
+    __syncthreads();
+    // ---- mix the heads, mask
+    for (int e = tid; e < R * PAGE; e += 256) {
+      const int kj = e % PAGE, r = e / PAGE, qi = r % BQ, h = r / BQ;
+      float s;
+      if (mix) {
+        s = 0.f;
+        for (int g = 0; g < H; ++g) s += mixs[h * H + g] * S1[((size_t)g * BQ + qi) * PAGE + kj];
+      } else {
+        s = S1[e];
+      }
+      const int dist = pos0 + qi - (jb + kj);
+      const bool ok = qi < nq && dist >= 0 && (window <= 0 || dist < window);
+      S2[e] = ok ? s : -INFINITY;
+    }
+    __syncthreads();
+    // ---- running maximum / denominator per (head, query) row: 32 lanes a row
+    for (int r = tid >> 5; r < R; r += 8) {
+      const float s = S2[(size_t)r * PAGE + (tid & 31)];
+      float mx = s;
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      const float m_old = mrow[r], m_new = fmaxf(m_old, mx);
+      const float p = expf(s - m_new);
+      float sum = p;
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+      S2[(size_t)r * PAGE + (tid & 31)] = p;
+      if ((tid & 31) == 0) {
+        const float cf = expf(m_old - m_new);
+        corr[r] = cf;
+        lrow[r] = lrow[r] * cf + sum;
+        mrow[r] = m_new;
+      }
+    }
+    // ---- weights x values
+    for (int c = 0; c < G; ++c) {
+      __syncthreads();  // Vt free; weights and corr visible
+      const T* vp = vcache + ((page * G + c) * PAGE) * V;
+      for (int i = tid; i < PAGE * V; i += 256) Vt[i] = (jb + i / V < j_hi) ? ldf<T>(vp, i) : 0.f;
+      __syncthreads();
+      for (int o = tid; o < rep * BQ * V; o += 256) {
+        const int v = o % V, rr = o / V;
+        const int r = c * rep * BQ + rr;  // (head, query) row: heads of this group are consecutive
+        const float* pw = S2 + (size_t)r * PAGE;
+        float a = acc[(size_t)r * V + v] * corr[r];
+#pragma unroll 8
+        for (int kj = 0; kj < PAGE; ++kj) a += pw[kj] * Vt[kj * V + v];
+        acc[(size_t)r * V + v] = a;
+      }
+    }
+  }
+  __syncthreads();
+  for (int o = tid; o < R * V; o += 256) {
+    const int v = o % V, r = o / V, qi = r % BQ, h = r / BQ;
+    if (qi >= nq) continue;
+    const size_t tok = (size_t)(q0 + t0 + qi);
+    if (nsplit == 1) {
+      const float l = lrow[r];
+      stf<T>(out, (tok * H + h) * V + v, l > 0.f ? acc[o] / l : 0.f);
+    } else {
+      part_acc[((tok * nsplit + split) * H + h) * V + v] = acc[o];
+      if (v == 0) {
+        part_ml[((tok * nsplit + split) * H + h) * 2] = mrow[r];
+        part_ml[((tok * nsplit + split) * H + h) * 2 + 1] = lrow[r];
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) window_attn_combine_kernel(const float* __restrict__ part_acc,
+                                                                   const float* __restrict__ part_ml,
+                                                                   T* __restrict__ out, int H, int V, int nsplit) {
+  const size_t tok = blockIdx.x;
+  for (int o = threadIdx.x; o < H * V; o += 256) {
+    const int h = o / V, v = o % V;
+    float M = -1e30f;
+    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[((tok * nsplit + s) * H + h) * 2]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float w = expf(part_ml[((tok * nsplit + s) * H + h) * 2] - M);
+      num += w * part_acc[((tok * nsplit + s) * H + h) * V + v];
+      den += w * part_ml[((tok * nsplit + s) * H + h) * 2 + 1];
+    }
+    stf<T>(out, (tok * H + h) * V + v, den > 0.f ? num / den : 0.f);
+  }
+}
+
+}  // namespace
+
+extern "C" int areal_qk_norm_cache_write(const void* proj, int64_t row_stride, const void* qw, const void* kw,
+                                         const int64_t* slots, void* q_out, void* kcache, void* vcache, int T, int H,
+                                         int G, int D, int V, float eps, int dt, hipStream_t st) {
+  if (T == 0) return 0;
+  if (dt == 0)
+    hipLaunchKernelGGL(qk_norm_cache_write_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)proj, row_stride,
+                       (const bf16_t*)qw, (const bf16_t*)kw, slots, (bf16_t*)q_out, (bf16_t*)kcache, (bf16_t*)vcache,
+                       H, G, D, V, eps);
+  else
+    hipLaunchKernelGGL(qk_norm_cache_write_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)proj, row_stride,
+                       (const float*)qw, (const float*)kw, slots, (float*)q_out, (float*)kcache, (float*)vcache, H, G,
+                       D, V, eps);
+  return (int)hipGetLastError();
+}
+
+// Largest query tile (16, 8, 4, 2, 1) whose LDS footprint fits the workgroup limit; 0 if even one query does not.
+extern "C" int areal_window_attn_tile(int H, int G, int D, int V, int want) {
+  for (int bq = want; bq >= 1; bq >>= 1) {
+    AttnShape sh{H, G, D, V, bq};
+    if (sh.floats() * sizeof(float) <= 156 * 1024) return bq;
+  }
+  return 0;
+}
+
+// B rows; row b's queries are tokens cu_q[b] .. cu_q[b+1] of q [T, H, D]; max_q = longest row. nsplit > 1 needs
+// part_acc [T, nsplit, H, V] and part_ml [T, nsplit, H, 2] (fp32) and is meant for single-query rows.
+extern "C" int areal_window_attn(const void* q, const void* kcache, const void* vcache, const int* block_tables,
+                                 int max_pages, const int* cu_q, const int* ctx_len, const void* mix, void* out,
+                                 float* part_acc, float* part_ml, int B, int max_q, int T, int H, int G, int D, int V,
+                                 int bq, float scale, float softcap, float slope_exp, int window, int sink, int nsplit,
+                                 int dt, hipStream_t st) {
+  if (B == 0 || T == 0) return 0;
+  if (G <= 0 || H % G != 0 || bq <= 0 || nsplit < 1) return -1;
+  AttnShape sh{H, G, D, V, bq};
+  const size_t lds = sh.floats() * sizeof(float);
+  if (lds > 160 * 1024) return -2;
+  if (nsplit > 1 && (!part_acc || !part_ml)) return -3;
+  const dim3 grid((max_q + bq - 1) / bq, B, nsplit);
+#define LAUNCH(TT)                                                                                                   \
+  do {                                                                                                               \
+    if (lds > 64 * 1024)                                                                                             \
+      HIP_RET(hipFuncSetAttribute((const void*)window_attn_kernel<TT>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                                  (int)lds));                                                                        \
+    hipLaunchKernelGGL(window_attn_kernel<TT>, grid, dim3(256), lds, st, (const TT*)q, (const TT*)kcache,            \
+                       (const TT*)vcache, block_tables, max_pages, cu_q, ctx_len, (const TT*)mix, (TT*)out, part_acc, \
+                       part_ml, sh, scale, softcap, slope_exp, window, sink, nsplit);                                \
+    if (nsplit > 1)                                                                                                  \
+      hipLaunchKernelGGL(window_attn_combine_kernel<TT>, dim3(T), dim3(256), 0, st, part_acc, part_ml, (TT*)out, H, \
+                         V, nsplit);                                                                                 \
+  } while (0)
+  if (dt == 0) LAUNCH(bf16_t);
+  else LAUNCH(float);
+#undef LAUNCH
+  return (int)hipGetLastError();
+}

@@ -39,6 +39,7 @@ static py::dict plan_to_dict(const Plan& p) {
   d["frequency_penalty"] = to_np(p.frequency_penalty);
   d["presence_penalty"] = to_np(p.presence_penalty);
   d["penalty_slot"] = to_np(p.penalty_slot);
+  d["state_slots"] = to_np(p.state_slots);
   if (p.kind == 1) {
     d["cu_q"] = to_np(p.cu_q);
     d["cu_k"] = to_np(p.cu_k);
@@ -135,6 +136,11 @@ class PyScheduler {
       throw std::runtime_error("process_decode: expected [n_steps, >=batch] outputs");
     s_.process_decode(p, toks.data(), lps.data(), (int)toks.shape(1), successor_in_flight);
   }
+  py::dict plan_replay(const std::vector<int64_t>& ids, const std::vector<std::vector<int32_t>>& toks, bool decode) {
+    if (ids.size() != toks.size()) throw std::runtime_error("plan_replay: one token list per request");
+    return remember(s_.plan_replay(ids, toks, decode));
+  }
+  void process_replay(int64_t plan_id) { s_.process_replay(take(plan_id)); }
   py::list take_finished() {
     py::list out;
     for (auto& f : s_.take_finished()) {
@@ -245,7 +251,9 @@ PYBIND11_MODULE(_runtime, m) {
       .def_readwrite("decode_steps", &SchedulerConfig::decode_steps)
       .def_readwrite("enable_prefix_cache", &SchedulerConfig::enable_prefix_cache)
       .def_readwrite("policy", &SchedulerConfig::policy)
-      .def_readwrite("schedule_conservativeness", &SchedulerConfig::schedule_conservativeness);
+      .def_readwrite("schedule_conservativeness", &SchedulerConfig::schedule_conservativeness)
+      .def_readwrite("num_state_slots", &SchedulerConfig::num_state_slots)
+      .def_readwrite("paged_prefill", &SchedulerConfig::paged_prefill);
   py::class_<PyScheduler>(m, "Scheduler")
       .def(py::init<const SchedulerConfig&>())
       .def("add_request", &PyScheduler::add_request, py::arg("rid"), py::arg("prompt"), py::arg("max_new_tokens"),
@@ -261,6 +269,11 @@ PYBIND11_MODULE(_runtime, m) {
       .def("process_decode", &PyScheduler::process_decode, py::arg("tokens"), py::arg("logprobs"),
            py::arg("plan_id") = -1, py::arg("successor_in_flight") = false)
       .def("take_finished", &PyScheduler::take_finished)
+      .def("open_replay", [](PyScheduler& s, const std::string& rid) { return s.s_.open_replay(rid); })
+      .def("plan_replay", &PyScheduler::plan_replay, py::arg("req_ids"), py::arg("tokens"), py::arg("decode") = false)
+      .def("process_replay", &PyScheduler::process_replay, py::arg("plan_id") = -1)
+      .def("close_replay", [](PyScheduler& s, int64_t id) { return s.s_.close_replay(id); })
+      .def("num_free_state_slots", [](PyScheduler& s) { return s.s_.num_free_state_slots(); })
       .def("progress",
            [](PyScheduler& s, int64_t id, int from) -> py::object {
              std::vector<int32_t> t, v;

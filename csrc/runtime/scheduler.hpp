@@ -22,7 +22,13 @@
 //     generated so far with finish reason "abort", their pages are released and the prefix cache is
 //     flushed; the client re-issues prompt+partial output and the KV is recomputed by prefill under
 //     the new weights,
-//   * every generated token is tagged with the weight version that produced it.
+//   * every generated token is tagged with the weight version that produced it,
+//   * models with recurrent layers: every admitted request owns one STATE SLOT (`num_state_slots`) from admission
+//     until its pages are released; plans carry the rows' slots. A slot is never cleared: the model starts a row
+//     whose first token has position 0 from the zero state,
+//   * replay requests (`open_replay` / `plan_replay` / `close_replay`): the client supplies every token, portion by
+//     portion, and reads logits at chosen places; nothing is sampled. Portions of several tokens (or a request's
+//     first token) form a prefill plan, single tokens of requests with context a one-step decode plan.
 #pragma once
 #include <algorithm>
 #include <chrono>
@@ -70,6 +76,8 @@ struct Request {
   double t_arrive = 0, t_first = 0, t_last = 0, t_finish = 0;
   std::vector<float> itl;
   int n_preempted = 0;
+  int state_slot = -1;          // slot of the recurrent state (models that have one)
+  bool replay = false;          // tokens come from the client, nothing is sampled
   int n_generated() const { return (int)tokens.size() - prompt_len; }
 };
 
@@ -108,6 +116,7 @@ struct Plan {
   std::vector<int32_t> min_remaining;  // tokens until stop tokens count (min_new_tokens)
   std::vector<int32_t> stop_ids;       // [B, MAX_DEVICE_STOP_IDS], -1 padded
   std::vector<int32_t> kill;           // continuation: 1 = the row's request is gone, deactivate it
+  std::vector<int32_t> state_slots;    // both kinds, per row: the request's recurrent-state slot (-1: the model has none)
   // sampling (both kinds)
   std::vector<float> temperature, top_p, frequency_penalty, presence_penalty;
   std::vector<int32_t> top_k, penalty_slot;
@@ -122,6 +131,8 @@ struct SchedulerConfig {
   bool enable_prefix_cache = true;
   std::string policy = "fcfs";  // "fcfs" | "lpm"
   float schedule_conservativeness = 1.0f;
+  int num_state_slots = 0;     // > 0: the model carries recurrent state, one slot per admitted request
+  bool paged_prefill = false;  // prefill plans always carry page tables (attention that reads the pages only)
 };
 
 inline double now_s() {
@@ -131,7 +142,9 @@ inline double now_s() {
 class Scheduler {
  public:
   explicit Scheduler(const SchedulerConfig& cfg)
-      : cfg_(cfg), bm_(cfg.num_pages, cfg.enable_prefix_cache) {}
+      : cfg_(cfg), bm_(cfg.num_pages, cfg.enable_prefix_cache) {
+    for (int i = cfg.num_state_slots - 1; i >= 0; --i) free_slots_.push_back(i);
+  }
 
   int64_t add_request(const std::string& rid, const std::vector<int32_t>& prompt, const SamplingParams& sp) {
     auto r = std::make_unique<Request>();
@@ -222,7 +235,7 @@ class Scheduler {
   // ------------------------------------------------------------------------------ planning
   bool prefill_possible() const {
     return !paused_ && (!prefilling_.empty() ||
-                        (!waiting_.empty() &&
+                        (!waiting_.empty() && (cfg_.num_state_slots == 0 || !free_slots_.empty()) &&
                          (int)(running_.size() + prefilling_.size()) < cfg_.max_running_requests));
   }
 
@@ -322,6 +335,81 @@ class Scheduler {
     sweep_finished(successor_in_flight);
   }
 
+  // ------------------------------------------------------------------------- replay of given tokens
+  // Admit a request that will be fed token by token. Returns -1 when every state slot is taken.
+  int64_t open_replay(const std::string& rid) {
+    if (cfg_.num_state_slots > 0 && free_slots_.empty()) return -1;
+    auto r = std::make_unique<Request>();
+    r->id = next_id_++;
+    r->rid = rid;
+    r->replay = true;
+    r->state = ReqState::RUNNING;
+    r->t_arrive = now_s();
+    if (cfg_.num_state_slots > 0) {
+      r->state_slot = free_slots_.back();
+      free_slots_.pop_back();
+    }
+    int64_t id = r->id;
+    reqs_[id] = std::move(r);
+    return id;
+  }
+
+  // One plan that feeds `toks[i]` to replay request `ids[i]`. `decode`: every portion is ONE token of a request that
+  // has context (a one-step decode plan); otherwise a prefill plan over the portions. Kind 0 (nothing is changed)
+  // when the page pool cannot hold the new tokens. The plan's results are booked with `process_replay`.
+  Plan plan_replay(const std::vector<int64_t>& ids, const std::vector<std::vector<int32_t>>& toks, bool decode) {
+    Plan p;
+    p.plan_id = next_plan_++;
+    int need_total = 0;
+    for (size_t i = 0; i < ids.size(); ++i) {
+      auto it = reqs_.find(ids[i]);
+      if (it == reqs_.end() || !it->second->replay || toks[i].empty()) return p;
+      const Request& r = *it->second;
+      if (decode && (toks[i].size() != 1 || r.tokens.empty())) return p;
+      if ((int)(r.tokens.size() + toks[i].size()) > cfg_.context_length) return p;
+      need_total += std::max(0, pages_for((int)(r.tokens.size() + toks[i].size())) - (int)r.pages.size());
+    }
+    if (ids.empty() || need_total > bm_.num_free()) return p;
+    std::vector<std::pair<int64_t, int>> rows;
+    for (size_t i = 0; i < ids.size(); ++i) {
+      Request& r = *reqs_[ids[i]];
+      r.tokens.insert(r.tokens.end(), toks[i].begin(), toks[i].end());
+      int need = pages_for((int)r.tokens.size()) - (int)r.pages.size();
+      if (need > 0) bm_.allocate(need, r.pages);
+      rows.emplace_back(ids[i], (int)r.tokens.size());
+    }
+    if (decode) {
+      p.kind = 2;
+      p.n_steps = 1;
+      emit_decode_rows(p, ids);
+    } else {
+      p.kind = 1;
+      p.cu_q.push_back(0);
+      p.cu_k.push_back(0);
+      for (auto& [id, end] : rows) emit_prefill_rows(p, *reqs_[id], end);
+      fill_prefill_tables(p, rows);
+    }
+    return p;
+  }
+
+  void process_replay(const Plan& p) {
+    for (auto id : p.req_ids) {
+      auto it = reqs_.find(id);
+      if (it != reqs_.end()) it->second->num_cached = (int)it->second->tokens.size();
+    }
+  }
+
+  // The request is over: its pages and its state slot return to the pools.
+  bool close_replay(int64_t id) {
+    auto it = reqs_.find(id);
+    if (it == reqs_.end() || !it->second->replay) return false;
+    release_pages(*it->second, false);
+    reqs_.erase(it);
+    return true;
+  }
+
+  int num_free_state_slots() const { return (int)free_slots_.size(); }
+
   std::vector<FinishedRequest> take_finished() {
     std::vector<FinishedRequest> out;
     out.swap(finished_);
@@ -378,8 +466,9 @@ class Scheduler {
     p.max_k = std::max(p.max_k, end);
     p.req_ids.push_back(r.id);
     p.chunk_end.push_back(end);
-    p.sample.push_back(end == n ? 1 : 0);
-    if (start > 0) p.has_prefix = true;
+    p.sample.push_back(end == n && !r.replay ? 1 : 0);
+    p.state_slots.push_back(r.state_slot);
+    if (start > 0 || cfg_.paged_prefill) p.has_prefix = true;
     fill_sampling(p, r, end == n);
   }
 
@@ -401,6 +490,7 @@ class Scheduler {
     if (cfg_.policy == "lpm" && waiting_.size() > 1) sort_waiting_lpm();
     while (budget > 0 && !waiting_.empty() &&
            (int)(running_.size() + prefilling_.size()) < cfg_.max_running_requests) {
+      if (cfg_.num_state_slots > 0 && free_slots_.empty()) break;  // every state slot is taken: wait for one
       int64_t id = waiting_.front();
       Request& r = *reqs_[id];
       int n = (int)r.tokens.size();
@@ -432,6 +522,10 @@ class Scheduler {
       }
       waiting_.pop_front();
       r.pages = std::move(pages);
+      if (cfg_.num_state_slots > 0) {
+        r.state_slot = free_slots_.back();
+        free_slots_.pop_back();
+      }
       r.num_cached = matched;
       r.state = ReqState::PREFILLING;
       prefilling_.push_back(id);
@@ -444,18 +538,7 @@ class Scheduler {
     if (rows.empty()) return;
     p.kind = 1;
     for (auto& [id, end] : rows) emit_prefill_rows(p, *reqs_[id], end);
-    if (p.has_prefix) {
-      // some row attends to context that is in the cache already (a reused prefix, earlier chunks): the attention
-      // kernel reads every row's context through its page table
-      p.max_pages = pages_for(p.max_k);
-      p.block_tables.assign(rows.size() * (size_t)p.max_pages, 0);
-      size_t row = 0;
-      for (auto& [id, end] : rows) {
-        Request& r = *reqs_[id];
-        std::copy(r.pages.begin(), r.pages.begin() + pages_for(end), p.block_tables.begin() + row * p.max_pages);
-        ++row;
-      }
-    }
+    fill_prefill_tables(p, rows);
     // rows whose last chunk is in this plan start decoding after it
     for (auto& [id, end] : rows) {
       Request& r = *reqs_[id];
@@ -464,6 +547,49 @@ class Scheduler {
         r.state = ReqState::RUNNING;
         running_.push_back(id);
       }
+    }
+  }
+
+  // some row attends to context that is in the cache already (a reused prefix, earlier chunks), or the model's
+  // attention reads the pages only: the kernel reaches every row's context through its page table
+  void fill_prefill_tables(Plan& p, const std::vector<std::pair<int64_t, int>>& rows) {
+    if (!p.has_prefix) return;
+    p.max_pages = pages_for(p.max_k);
+    p.block_tables.assign(rows.size() * (size_t)p.max_pages, 0);
+    size_t row = 0;
+    for (auto& [id, end] : rows) {
+      Request& r = *reqs_[id];
+      std::copy(r.pages.begin(), r.pages.begin() + pages_for(end), p.block_tables.begin() + row * p.max_pages);
+      ++row;
+    }
+  }
+
+  // Rows of a one- or multi-step decode plan for the given requests (each consumes its last token).
+  void emit_decode_rows(Plan& p, const std::vector<int64_t>& ids) {
+    int max_pages = 0;
+    for (auto id : ids) max_pages = std::max(max_pages, (int)reqs_[id]->pages.size());
+    p.max_pages = max_pages;
+    p.block_tables.assign(ids.size() * (size_t)max_pages, 0);
+    p.stop_ids.assign(ids.size() * (size_t)MAX_DEVICE_STOP_IDS, -1);
+    size_t row = 0;
+    for (auto id : ids) {
+      Request& r = *reqs_[id];
+      int pos = (int)r.tokens.size() - 1;
+      p.req_ids.push_back(id);
+      p.input_ids.push_back(r.tokens.back());
+      p.positions.push_back(pos);
+      p.context_lens.push_back(pos + 1);
+      p.slot_mapping.push_back((int64_t)r.pages[pos / PAGE] * PAGE + pos % PAGE);
+      std::copy(r.pages.begin(), r.pages.end(), p.block_tables.begin() + row * max_pages);
+      p.remaining.push_back(r.replay ? (1 << 30) : std::max(
+          1, std::min(r.sp.max_new_tokens - r.n_generated(), cfg_.context_length - (int)r.tokens.size())));
+      p.min_remaining.push_back(std::max(0, r.sp.min_new_tokens - r.n_generated()));
+      for (size_t j = 0; j < r.sp.stop_token_ids.size() && j < (size_t)MAX_DEVICE_STOP_IDS; ++j)
+        p.stop_ids[row * MAX_DEVICE_STOP_IDS + j] = r.sp.stop_token_ids[j];
+      p.kill.push_back(0);
+      p.state_slots.push_back(r.state_slot);
+      fill_sampling(p, r);
+      ++row;
     }
   }
 
@@ -487,30 +613,7 @@ class Scheduler {
     if (running_.empty()) return;
     p.kind = 2;
     p.n_steps = k;
-    int max_pages = 0;
-    for (auto id : running_) max_pages = std::max(max_pages, (int)reqs_[id]->pages.size());
-    p.max_pages = max_pages;
-    p.block_tables.assign(running_.size() * (size_t)max_pages, 0);
-    p.stop_ids.assign(running_.size() * (size_t)MAX_DEVICE_STOP_IDS, -1);
-    size_t row = 0;
-    for (auto id : running_) {
-      Request& r = *reqs_[id];
-      int pos = (int)r.tokens.size() - 1;
-      p.req_ids.push_back(id);
-      p.input_ids.push_back(r.tokens.back());
-      p.positions.push_back(pos);
-      p.context_lens.push_back(pos + 1);
-      p.slot_mapping.push_back((int64_t)r.pages[pos / PAGE] * PAGE + pos % PAGE);
-      std::copy(r.pages.begin(), r.pages.end(), p.block_tables.begin() + row * max_pages);
-      p.remaining.push_back(std::max(
-          1, std::min(r.sp.max_new_tokens - r.n_generated(), cfg_.context_length - (int)r.tokens.size())));
-      p.min_remaining.push_back(std::max(0, r.sp.min_new_tokens - r.n_generated()));
-      for (size_t j = 0; j < r.sp.stop_token_ids.size() && j < (size_t)MAX_DEVICE_STOP_IDS; ++j)
-        p.stop_ids[row * MAX_DEVICE_STOP_IDS + j] = r.sp.stop_token_ids[j];
-      p.kill.push_back(0);
-      fill_sampling(p, r);
-      ++row;
-    }
+    emit_decode_rows(p, running_);
   }
 
   void preempt_last() {
@@ -604,10 +707,15 @@ class Scheduler {
     deferred_.clear();
   }
 
+  // Pages and the state slot go back together: whatever may still write the one may still write the other.
   void release_pages(Request& r, bool publish) {
-    if (publish && r.num_cached > 0) bm_.publish(r.tokens.data(), r.num_cached, r.pages);
+    if (publish && r.num_cached > 0 && !r.replay) bm_.publish(r.tokens.data(), r.num_cached, r.pages);
     bm_.release_all(r.pages);
     r.pages.clear();
+    if (r.state_slot >= 0) {
+      free_slots_.push_back(r.state_slot);
+      r.state_slot = -1;
+    }
   }
 
   void finish(Request& r) {
@@ -635,6 +743,7 @@ class Scheduler {
   std::vector<int64_t> running_;
   std::vector<std::unique_ptr<Request>> deferred_;  // finished, pages still possibly written by the device
   std::vector<FinishedRequest> finished_;
+  std::vector<int> free_slots_;  // recurrent-state slots not owned by a request
   int64_t next_id_ = 1, next_plan_ = 1;
   bool paused_ = false;
   int version_ = 0;
