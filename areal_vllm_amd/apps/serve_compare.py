@@ -1,0 +1,105 @@
+"""Serving throughput of a layer-list design beside the closest standard transformer of equal size.
+
+For every size a Kuzanex model (window attention : mLSTM layers 1 : 2, xIELU feed-forward) and a Qwen3-style
+transformer (grouped-query attention with q/k norm, gated MLP) of the same width, depth, head layout and - through
+the width of its MLP - parameter count are served by the rollout engine on random weights: the same prompts, the same
+number of new tokens, prefill plans and captured decode graphs. Reported per model: prompt tokens/s over the prefill
+plans and generated tokens/s over the decode plans (the engine's own clocks), and the parameters per token.
+"""
+import json
+import sys
+import time
+from typing import Any, Dict, List
+
+import torch
+
+SIZES = {
+    # name: width, layers, heads, kv heads, head size, feed-forward, window
+    "w1024": (1024, 6, 8, 2, 128, 4096, 512),
+    "w2048": (2048, 6, 16, 4, 128, 8192, 512),
+    "w4096": (4096, 3, 32, 8, 128, 14336, 1024),
+}
+VOCAB = 32768
+
+
+def kuzanex_dict(width, layers, heads, kv, dim, ff, window) -> Dict[str, Any]:
+    ls = []
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": ff}
+        if i % 3 == 0:
+            ls.append({"type": "attention", "mlp": mlp,
+                       "mixer": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                 "softcap": 30.0, "mask": {"size": window}}})
+        else:
+            ls.append({"type": "mlstm", "mlp": mlp,
+                       "mixer": {"heads": heads // 2, "dim": dim, "vdim": 2 * dim, "gate_cap": 12.0}})
+    return {"architecture": "Kuzanex", "layers": ls, "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "vocab": VOCAB,
+            "width": width}
+
+
+def twin_config(kcfg, width, layers, heads, kv, dim):
+    """Qwen3-style transformer whose gated MLP is as wide as the parameter budget of the Kuzanex model allows."""
+    from ..models.config import ModelConfig
+
+    body = kcfg.n_params(with_embedding=False)
+    attn = width * (heads + 2 * kv) * dim + width * heads * dim
+    inter = max(64, int(round((body / layers - attn) / (3 * width) / 64)) * 64)
+    return ModelConfig(family="qwen3", vocab_size=VOCAB, hidden_size=width, n_layers=layers, n_q_heads=heads,
+                       n_kv_heads=kv, head_dim=dim, intermediate_size=inter, tie_word_embeddings=False, qkv_bias=False,
+                       qk_norm=True, rope_theta=1e6, max_position_embeddings=8192, rms_norm_eps=1e-6)
+
+
+def measure(cfg, n_prompts: int, prompt_len: int, new_tokens: int, device) -> Dict[str, float]:
+    from ..api.cli_args import InferenceServerConfig
+    from ..inference.engine import NativeInferenceEngine
+    from ..ops.attention import PAGE_SIZE
+
+    ctx = prompt_len + new_tokens + PAGE_SIZE
+    srv = InferenceServerConfig(model_path="", dtype="bfloat16", context_length=ctx, max_running_requests=n_prompts,
+                                num_continuous_decode_steps=8, max_prefill_tokens=8192, disable_radix_cache=True)
+    pages = n_prompts * ((ctx + PAGE_SIZE - 1) // PAGE_SIZE + 1) + 8
+    eng = NativeInferenceEngine(srv, model_config=cfg, device=device, num_pages=pages)
+    eng.initialize(load_weights=False)
+    g = torch.Generator().manual_seed(7)
+    out = {}
+    try:
+        for phase in ("warmup", "timed"):
+            prompts = [torch.randint(3, VOCAB, (prompt_len,), generator=g).tolist() for _ in range(n_prompts)]
+            before = dict(eng.stats)
+            p0 = eng.sched.total_prompt_tokens()
+            t0 = time.perf_counter()
+            res = eng.generate_blocking(prompts, max_new_tokens=new_tokens, temperature=1.0)
+            wall = time.perf_counter() - t0
+            gen = sum(len(r.output_tokens) for r in res)
+            pt = eng.stats["prefill_time"] - before["prefill_time"]
+            dt = eng.stats["decode_time"] - before["decode_time"]
+            out = dict(prefill_tok_s=(eng.sched.total_prompt_tokens() - p0) / max(pt, 1e-9),
+                       decode_tok_s=(gen - n_prompts) / max(dt, 1e-9), wall_s=wall,
+                       prefill_ms=1e3 * pt, decode_ms=1e3 * dt)
+    finally:
+        eng.destroy()
+    return out
+
+
+def run(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, device="cuda") -> int:
+    from ..models.config import ModelConfig
+
+    dev = torch.device(device, 0) if device == "cuda" else torch.device(device)
+    for name in sizes:
+        width, layers, heads, kv, dim, ff, window = SIZES[name]
+        kcfg = ModelConfig.from_hf_dict(kuzanex_dict(width, layers, heads, kv, dim, ff, window))
+        tcfg = twin_config(kcfg, width, layers, heads, kv, dim)
+        row = {"size": name, "width": width, "layers": layers, "heads": heads, "kv_heads": kv, "head_dim": dim,
+               "window": window, "prompts": n_prompts, "prompt_len": prompt_len, "new_tokens": new_tokens,
+               "dtype": "bf16", "data": "synthetic"}
+        for label, cfg in (("kuzanex", kcfg), ("qwen3_twin", tcfg)):
+            m = measure(cfg, n_prompts, prompt_len, new_tokens, dev)
+            row[label] = {"params_no_embedding": cfg.n_params(with_embedding=False), **{k: round(v, 1) for k, v in m.items()}}
+        row["prefill_ratio"] = round(row["kuzanex"]["prefill_tok_s"] / row["qwen3_twin"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row["kuzanex"]["decode_tok_s"] / row["qwen3_twin"]["decode_tok_s"], 3)
+        print(json.dumps(row), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(run(sys.argv[1:] or list(SIZES), 32, 1024, 64))

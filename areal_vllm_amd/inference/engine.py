@@ -71,6 +71,8 @@ class NativeInferenceEngine:
         self.config = config
         self.device = device or (torch.device("cuda", torch.cuda.current_device()) if torch.cuda.is_available()
                                  else torch.device("cpu"))
+        if self.device.type == "cuda" and self.device.index is None:  # the loop thread binds itself to an index
+            self.device = torch.device("cuda", torch.cuda.current_device())
         self.dtype = getattr(torch, config.dtype)
         from ..engine.train_engine import _resolve_model_config
 
@@ -241,11 +243,8 @@ class NativeInferenceEngine:
             torch.cuda.set_device(self.device)
             # the engine owns a stream: decode graphs overlap with whatever the trainer thread runs on
             # its stream (colocated asynchronous training)
-            # high priority: decode kernels are small (a few hundred workgroups) and latency-bound; when the
-            # trainer's large GEMMs share the GPU they would otherwise queue behind full-chip grids, while with
-            # priority they take the CUs they need and the trainer's grids fill the rest
-            prio = int(os.environ.get("AREAL_ROLLOUT_STREAM_PRIORITY", "-1"))
-            self._stream = torch.cuda.Stream(device=self.device, priority=prio)
+            # (default priority: streams of different priorities are not mixed in one process)
+            self._stream = torch.cuda.Stream(device=self.device)
             torch.cuda.set_stream(self._stream)
         try:
             while not self._stop.is_set():

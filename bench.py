@@ -100,6 +100,11 @@ def parse_args():
     p.add_argument("--decoupled-steps", type=int, default=8, help="timed steps of that second pass (at most --steps)")
     p.add_argument("--decoupled-budget", type=float, default=300.0,
                    help="seconds the second pass may take before it is ended and reported as an error")
+    p.add_argument("--serve-compare", default="", metavar="SIZES",
+                   help="instead of the RL step: serving throughput (prefill and decode tokens/s) of the Kuzanex design "
+                        "beside a Qwen3-style transformer of equal size, one JSON line per size; comma-separated names "
+                        "out of w1024, w2048, w4096, or 'all' (--prompts-per-gpu prompts of --prompt-len-max tokens, "
+                        "--max-new-tokens new tokens each)")
     a = p.parse_args()
     if a.seq_len:
         a.max_new_tokens = a.seq_len - a.prompt_len_max
@@ -272,6 +277,11 @@ def launch_ranks(args):
 
 def main():
     args = parse_args()
+    if args.serve_compare:
+        from areal_vllm_amd.apps import serve_compare
+
+        names = list(serve_compare.SIZES) if args.serve_compare == "all" else args.serve_compare.split(",")
+        sys.exit(serve_compare.run(names, args.prompts_per_gpu, args.prompt_len_max, args.max_new_tokens, args.device))
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ and "RANK" not in os.environ:
         sys.exit(launch_ranks(args))
     run_rank(args)

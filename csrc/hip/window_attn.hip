@@ -128,8 +128,6 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
   const int p_lo = j_lo / PAGE, p_hi = (j_hi + PAGE - 1) / PAGE;
   const int per = (p_hi - p_lo + nsplit - 1) / nsplit;
   const int my_lo = p_lo + split * per, my_hi = min(p_hi, my_lo + per);
-  const float log2e_unused = 0.f;
-  (void)log2e_unused;
 
   for (int pg = my_lo; pg < my_hi; ++pg) {
     const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
@@ -283,9 +281,12 @@ extern "C" int areal_window_attn(const void* q, const void* kcache, const void* 
   const dim3 grid((max_q + bq - 1) / bq, B, nsplit);
 #define LAUNCH(TT)                                                                                                   \
   do {                                                                                                               \
-    if (lds > 64 * 1024)                                                                                             \
+    static size_t allowed = 64 * 1024; /* raised once per size: no attribute call inside a stream capture */         \
+    if (lds > allowed) {                                                                                             \
       HIP_RET(hipFuncSetAttribute((const void*)window_attn_kernel<TT>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
-                                  (int)lds));                                                                        \
+                                  160 * 1024));                                                                      \
+      allowed = 160 * 1024;                                                                                          \
+    }                                                                                                                \
     hipLaunchKernelGGL(window_attn_kernel<TT>, grid, dim3(256), lds, st, (const TT*)q, (const TT*)kcache,            \
                        (const TT*)vcache, block_tables, max_pages, cu_q, ctx_len, (const TT*)mix, (TT*)out, part_acc, \
                        part_ml, sh, scale, softcap, slope_exp, window, sink, nsplit);                                \
