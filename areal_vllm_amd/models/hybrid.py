@@ -139,9 +139,9 @@ class WindowAttentionMixer(nn.Module):
         proj = F.linear(xc, self.proj, self.proj_bias)
         q = wattn.qk_norm_cache_write(proj, self.q_norm, self.k_norm, st.slots, kc, vc, H, self.eps)
         o = wattn.window_attention(q, kc, vc, st.block_tables, st.cu_q, st.ctx_len, st.max_q, self.shape, self.talk,
-                                   nsplit=st.nsplit if st.max_q == 1 else 1, workspace=st.workspace)
-        gate = torch.sigmoid(proj[:, (H + G) * D + G * V:].float()).to(o.dtype)
-        return F.linear((o * gate.unsqueeze(-1)).view(T, H * V), self.o)
+                                   nsplit=st.nsplit if st.max_q == 1 else 1, workspace=st.workspace,
+                                   gate=proj[:, (H + G) * D + G * V:])
+        return F.linear(o.view(T, H * V), self.o)
 
 
 class MLSTMMixer(nn.Module):

@@ -76,9 +76,13 @@ def decode_splits(batch: int, window: int, max_context: int) -> int:
 def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_tables: torch.Tensor,
                      cu_q: torch.Tensor, ctx_len: torch.Tensor, max_q: int, shape: ScoreShape,
                      mix: Optional[torch.Tensor] = None, nsplit: int = 1,
-                     workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+                     workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                     gate: Optional[torch.Tensor] = None, matrix_cores: bool = True) -> torch.Tensor:
     """q [T, H, D] (row b owns tokens cu_q[b]:cu_q[b+1], the LAST positions of its context of ctx_len[b] tokens,
-    whose keys / values are in the cache already). mix [H, H] or None. Returns [T, H, Dv]."""
+    whose keys / values are in the cache already). mix [H, H] or None. gate [T, H] (a view with unit stride along
+    the heads) or None: head h of token t is multiplied by sigmoid(gate[t, h]). `matrix_cores`: bf16 rows of several
+    queries with head sizes 64 / 128 and at most 16 heads run the MFMA kernel (False: always the plain one).
+    Returns [T, H, Dv]."""
     T, H, D = q.shape
     G, V = kcache.shape[1], vcache.shape[3]
     B = cu_q.numel() - 1
@@ -86,6 +90,7 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         assert q.is_contiguous() and kcache.dtype == q.dtype and block_tables.dtype == torch.int32
         assert cu_q.dtype == torch.int32 and ctx_len.dtype == torch.int32 and block_tables.is_contiguous()
         assert mix is None or (mix.dtype == q.dtype and mix.is_contiguous() and mix.shape == (H, H))
+        assert gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and gate.shape == (T, H))
         out = torch.empty(T, H, V, dtype=q.dtype, device=q.device)
         want = 1 if max_q == 1 else 16
         while want > 1 and want // 2 >= max_q:
@@ -103,10 +108,11 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
             assert pa.numel() >= T * nsplit * H * V and pm.numel() >= T * nsplit * H * 2
         L.check(L.lib().areal_window_attn(
             L.ptr(q), L.ptr(kcache), L.ptr(vcache), L.ptr(block_tables), L.c_int(block_tables.shape[1]), L.ptr(cu_q),
-            L.ptr(ctx_len), L.ptr(mix), L.ptr(out), L.ptr(pa), L.ptr(pm), L.c_int(B), L.c_int(int(max_q)), L.c_int(T),
+            L.ptr(ctx_len), L.ptr(mix), L.ptr(gate), L.c_int64(gate.stride(0) if gate is not None else 0), L.ptr(out),
+            L.ptr(pa), L.ptr(pm), L.c_int(B), L.c_int(int(max_q)), L.c_int(T),
             L.c_int(H), L.c_int(G), L.c_int(D), L.c_int(V), L.c_int(bq), L.c_float(shape.scale),
             L.c_float(shape.softcap), L.c_float(shape.slope_exp), L.c_int(int(shape.window)), L.c_int(int(shape.sink)),
-            L.c_int(int(nsplit)), L.c_int(L.dtype_flag(q)), L.stream_ptr()), "window_attn")
+            L.c_int(int(nsplit)), L.c_int(L.dtype_flag(q)), L.c_int(int(matrix_cores)), L.stream_ptr()), "window_attn")
         return out
     out = torch.zeros(T, H, V, dtype=torch.float32, device=q.device)
     cq, cl = cu_q.tolist(), ctx_len.tolist()
@@ -137,4 +143,6 @@ def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         e = torch.exp(s - m)
         den = e.sum(-1, keepdim=True) + (torch.exp(-m) if shape.sink else 0.0)
         out[cq[b]:cq[b + 1]] = torch.einsum("hij,hjv->ihv", e / den, vv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float()).unsqueeze(-1)
     return out.to(q.dtype)

@@ -6,7 +6,7 @@
 //   t_h        = sum_g M[h, g] s_g                                 head mixing (M = null: t_h = s_h)
 //   visible:     0 <= i - j < window                               (window <= 0: every earlier key)
 //   p_h(j)     = exp(t_h(j)) / (sink + sum_j' exp(t_h(j')))        sink = 1: a key of score 0 that has no value
-//   o_h(i)     = sum_j p_h(j) v_c(h)(j)
+//   o_h(i)     = sum_j p_h(j) v_c(h)(j)  [* sigmoid(gate_h(i)) when a gate is given: one number per head and token]
 //
 // Scores, weights and the accumulation run in fp32 whatever the storage type T (bf16 / fp32) of q, the caches
 // and the output. Because the heads are mixed before the softmax, one workgroup owns ALL heads of a tile of BQ
@@ -14,7 +14,8 @@
 // denominator of every (head, query) row and accumulates p.v into LDS-resident fp32 accumulators.
 //
 // The same kernel serves prompt portions (tiles of BQ queries, grid x = tiles, y = rows of the batch) and
-// decoding (BQ = 1, grid z = splits of the visible key range whose partial results `window_attn_combine` merges).
+// decoding (BQ = 1, grid z = splits of the visible key range whose partial results `window_attn_combine` merges);
+// bf16 prompt portions of the common head sizes take the matrix-core kernel further down instead.
 // Queries of row b are the LAST cu_q[b+1] - cu_q[b] positions of its context of ctx_len[b] tokens.
 //
 // Cache layout: K [pages, G, 32, D], V [pages, G, 32, Dv], token-major inside a page.
@@ -85,8 +86,8 @@ template <typename T>
 __global__ void __launch_bounds__(256) window_attn_kernel(
     const T* __restrict__ q, const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
-    const int* __restrict__ ctx_len, const T* __restrict__ mix, T* __restrict__ out, float* __restrict__ part_acc,
-    float* __restrict__ part_ml, AttnShape sh, float scale, float softcap, float slope_exp, int window, int sink,
+    const int* __restrict__ ctx_len, const T* __restrict__ mix, const T* __restrict__ gate, int64_t gate_stride,
+    T* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, AttnShape sh, float scale, float softcap, float slope_exp, int window, int sink,
     int nsplit) {
   extern __shared__ float lds[];
   const int H = sh.H, G = sh.G, D = sh.D, V = sh.V, BQ = sh.BQ;
@@ -209,7 +210,9 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
     const size_t tok = (size_t)(q0 + t0 + qi);
     if (nsplit == 1) {
       const float l = lrow[r];
-      stf<T>(out, (tok * H + h) * V + v, l > 0.f ? acc[o] / l : 0.f);
+      float val = l > 0.f ? acc[o] / l : 0.f;
+      if (gate) val /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + h));
+      stf<T>(out, (tok * H + h) * V + v, val);
     } else {
       part_acc[((tok * nsplit + split) * H + h) * V + v] = acc[o];
       if (v == 0) {
@@ -220,9 +223,234 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// Matrix-core version for bf16 prompt portions (head sizes 64 / 128, up to 16 heads). One workgroup = 16 queries x
+// all heads, H / HPW waves, wave w owning heads w HPW .. w HPW + HPW - 1. Per 32-key page:
+//   stage   K of every key/value head -> LDS [G][32][D + 8], V transposed -> LDS [G][V][32 + 8]
+//   scores  per owned head: q (registers) x K^T, bf16 MFMA 16x16x32 with fp32 accumulation; scale, cap, distance bias
+//           in fp32 -> LDS SM[head][query][key] (fp32)
+//   mix     fp32 MFMA 16x16x4: M [16 x 16, zero padded] x SM[all heads][query, 16 keys]; a wave takes queries
+//           w, w + waves, ...; mask, running maximum / denominator per (head, query) in LDS; the weight p (fp32) goes
+//           back into its 4-byte slot of SM as the pair (bf16(p), bf16(p - bf16(p)))
+//   p.v     per owned head: bf16 MFMA over the (hi, lo) pairs as 32 k-slots against the value rows taken twice: the
+//           product carries 16 bits of p's mantissa (the values themselves are bf16), fp32 accumulation
+template <int HPW, int DK, int VT_, int MAXT>
+__global__ void __launch_bounds__(MAXT) window_attn_mfma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_len, const bf16_t* __restrict__ mix, const bf16_t* __restrict__ gate,
+    int64_t gate_stride, bf16_t* __restrict__ out, int H, int G, float scale, float softcap, float slope_exp,
+    int window, int sink) {
+  constexpr int D = DK * 32, V = VT_ * 16, KS = D + 8, VS = PAGE + 8, SS = PAGE + 4;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  unsigned* SM = reinterpret_cast<unsigned*>(smem);                      // [16][16][SS] 4-byte slots
+  bf16_t* KT = reinterpret_cast<bf16_t*>(smem + 16 * 16 * SS * 4);       // [G][32][KS]
+  bf16_t* VTt = KT + (size_t)G * PAGE * KS;                              // [G][V][VS]
+  float* mS = reinterpret_cast<float*>(VTt + (size_t)G * V * VS);        // [16][16]
+  float* lS = mS + 256;
+  float* cS = lS + 256;
+  float* Tm = cS + 256;                                                  // [16][16]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthr = blockDim.x, NW = nthr >> 6;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int b = blockIdx.y;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0, t0 = blockIdx.x * 16;
+  if (t0 >= qlen) return;
+  const int nq = min(16, qlen - t0), ctx = ctx_len[b], pos0 = ctx - qlen + t0, rep = H / G;
+
+  for (int i = tid; i < 16 * 16 * SS; i += nthr) SM[i] = 0u;
+  for (int i = tid; i < 256; i += nthr) {
+    mS[i] = sink ? 0.f : -1e30f;
+    lS[i] = sink ? 1.f : 0.f;
+    cS[i] = 1.f;
+    const int h = i >> 4, g = i & 15;
+    Tm[i] = (h < H && g < H) ? (mix ? bf2f(mix[h * H + g]) : (h == g ? 1.f : 0.f)) : 0.f;
+  }
+  bf16x8 qf[HPW][DK];
+  f32x4 acc[HPW][VT_];
+  float slope[HPW];
+#pragma unroll
+  for (int hh = 0; hh < HPW; ++hh) {
+    const int h = wave * HPW + hh;
+    slope[hh] = slope_exp != 0.f ? exp2f(-slope_exp * (float)(h + 1) / (float)H) : 0.f;
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks) {
+      if (r16 < nq) qf[hh][ks] = ld8(q + ((size_t)(q0 + t0 + r16) * H + h) * D + 32 * ks + 8 * quad);
+      else qf[hh][ks] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+    }
+#pragma unroll
+    for (int vt = 0; vt < VT_; ++vt) acc[hh][vt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+  const int j_hi = pos0 + nq;
+  const int j_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int p_lo = j_lo / PAGE, p_hi = (j_hi + PAGE - 1) / PAGE;
+  const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+
+  for (int pg = p_lo; pg < p_hi; ++pg) {
+    const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
+    const int jb = pg * PAGE;
+    __syncthreads();  // the page before is consumed (first time: the set-up above is visible)
+    for (int i = tid; i < G * PAGE * (D / 8); i += nthr) {
+      const int dv = i % (D / 8), key = (i / (D / 8)) % PAGE, c = i / (PAGE * (D / 8));
+      st8(KT + ((size_t)c * PAGE + key) * KS + 8 * dv, ld8(kcache + ((page * G + c) * PAGE + key) * D + 8 * dv));
+    }
+    for (int i = tid; i < G * PAGE * (V / 8); i += nthr) {
+      const int key = i % PAGE, vv = (i / PAGE) % (V / 8), c = i / (PAGE * (V / 8));
+      bf16x8 x = ld8(vcache + ((page * G + c) * PAGE + key) * V + 8 * vv);
+      const bool live = jb + key < j_hi;  // rows past the tile's last key may hold anything: they must not reach p.v
+#pragma unroll
+      for (int e = 0; e < 8; ++e) VTt[((size_t)c * V + 8 * vv + e) * VS + key] = live ? x[e] : (bf16_t)0.f;
+    }
+    __syncthreads();
+    // ---- shaped scores of the owned heads
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      const int h = wave * HPW + hh, c = h / rep;
+      f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < DK; ++ks) {
+        const bf16x8 b0 = ld8(KT + ((size_t)c * PAGE + r16) * KS + 32 * ks + 8 * quad);
+        const bf16x8 b1 = ld8(KT + ((size_t)c * PAGE + 16 + r16) * KS + 32 * ks + 8 * quad);
+        c0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[hh][ks], b0, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[hh][ks], b1, c1, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int qi = 4 * quad + i;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          float sc = (half ? c1[i] : c0[i]) * scale;
+          if (softcap > 0.f) {
+            const float e = __expf(2.f * fminf(fmaxf(sc * inv_cap, -15.f), 15.f));
+            sc = softcap * ((e - 1.f) / (e + 1.f));
+          }
+          sc -= slope[hh] * (float)(pos0 + qi - (jb + 16 * half + r16));
+          SM[((size_t)h * 16 + qi) * SS + 16 * half + r16] = __float_as_uint(sc);
+        }
+      }
+    }
+    __syncthreads();
+    // ---- mix the heads (fp32 matrix cores), mask, running softmax statistics, weights back into SM
+    for (int qi = wave; qi < 16; qi += NW) {
+      f32x4 m0 = {0.f, 0.f, 0.f, 0.f}, m1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const float a = Tm[r16 * 16 + 4 * kk + quad];
+        const float b0 = __uint_as_float(SM[((size_t)(4 * kk + quad) * 16 + qi) * SS + r16]);
+        const float b1 = __uint_as_float(SM[((size_t)(4 * kk + quad) * 16 + qi) * SS + 16 + r16]);
+        m0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b0, m0, 0, 0, 0);
+        m1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b1, m1, 0, 0, 0);
+      }
+      const int d0 = pos0 + qi - (jb + r16), d1 = d0 - 16;
+      const bool ok0 = qi < nq && d0 >= 0 && (window <= 0 || d0 < window);
+      const bool ok1 = qi < nq && d1 >= 0 && (window <= 0 || d1 < window);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int h = 4 * quad + i;
+        const float s0 = ok0 ? m0[i] : -INFINITY, s1 = ok1 ? m1[i] : -INFINITY;
+        float mx = fmaxf(s0, s1);
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float m_old = mS[h * 16 + qi], m_new = fmaxf(m_old, mx);
+        const float p0 = __expf(s0 - m_new), p1 = __expf(s1 - m_new);
+        float sum = p0 + p1;
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        if (h < H) {
+          const bf16_t h0 = f2bf(p0), h1 = f2bf(p1);
+          const bf16_t l0 = f2bf(p0 - bf2f(h0)), l1 = f2bf(p1 - bf2f(h1));
+          SM[((size_t)h * 16 + qi) * SS + r16] = (unsigned)__builtin_bit_cast(unsigned short, h0) |
+                                                 ((unsigned)__builtin_bit_cast(unsigned short, l0) << 16);
+          SM[((size_t)h * 16 + qi) * SS + 16 + r16] = (unsigned)__builtin_bit_cast(unsigned short, h1) |
+                                                      ((unsigned)__builtin_bit_cast(unsigned short, l1) << 16);
+          if (r16 == 0) {
+            const float cf = __expf(m_old - m_new);
+            cS[h * 16 + qi] = cf;
+            lS[h * 16 + qi] = lS[h * 16 + qi] * cf + sum;
+            mS[h * 16 + qi] = m_new;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    // ---- weights x values of the owned heads
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      const int h = wave * HPW + hh, c = h / rep;
+      f32x4 cf;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) cf[i] = cS[h * 16 + 4 * quad + i];
+#pragma unroll
+      for (int vt = 0; vt < VT_; ++vt) acc[hh][vt] *= cf;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(SM + ((size_t)h * 16 + r16) * SS + 16 * kb + 4 * quad);
+#pragma unroll
+        for (int vt = 0; vt < VT_; ++vt) {
+          const bf16x4 v4 =
+              *reinterpret_cast<const bf16x4*>(VTt + ((size_t)c * V + 16 * vt + r16) * VS + 16 * kb + 4 * quad);
+          const bf16x8 bb = {v4[0], v4[0], v4[1], v4[1], v4[2], v4[2], v4[3], v4[3]};
+          acc[hh][vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bb, acc[hh][vt], 0, 0, 0);
+        }
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int hh = 0; hh < HPW; ++hh) {
+    const int h = wave * HPW + hh;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int qi = 4 * quad + i;
+      if (qi >= nq) continue;
+      const size_t tok = (size_t)(q0 + t0 + qi);
+      const float l = lS[h * 16 + qi];
+      float f = l > 0.f ? 1.f / l : 0.f;
+      if (gate) f /= 1.f + expf(-bf2f(gate[tok * gate_stride + h]));
+#pragma unroll
+      for (int vt = 0; vt < VT_; ++vt) out[(tok * H + h) * V + 16 * vt + r16] = f2bf(acc[hh][vt][i] * f);
+    }
+  }
+}
+
+size_t mfma_lds_bytes(int G, int D, int V) {
+  return (size_t)16 * 16 * (PAGE + 4) * 4 + (size_t)G * PAGE * (D + 8) * 2 + (size_t)G * V * (PAGE + 8) * 2 + 4 * 256 * 4;
+}
+int mfma_heads_per_wave(int H) { return (H % 4 == 0 && H >= 16) ? 4 : ((H % 2 == 0 && H >= 8) ? 2 : 1); }
+bool mfma_usable(int H, int G, int D, int V) {
+  if (H > 16 || H < 1 || G < 1 || H % G != 0 || (D != 64 && D != 128) || (V != 64 && V != 128)) return false;
+  if (H / mfma_heads_per_wave(H) > 8) return false;
+  return mfma_lds_bytes(G, D, V) <= 160 * 1024;
+}
+
+template <int HPW, int MAXT>
+int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q, const bf16_t* kc, const bf16_t* vc,
+                const int* bt, int max_pages, const int* cu_q, const int* ctx_len, const bf16_t* mix,
+                const bf16_t* gate, int64_t gate_stride, bf16_t* out, int H, int G, int D, int V, float scale,
+                float softcap, float slope_exp, int window, int sink) {
+#define MFMA_CASE(DKV, VTV)                                                                                        \
+  do {                                                                                                             \
+    static bool raised = false; /* once per kernel: no attribute call inside a stream capture later */            \
+    if (!raised) {                                                                                                 \
+      HIP_RET(hipFuncSetAttribute((const void*)window_attn_mfma_kernel<HPW, DKV, VTV, MAXT>,                       \
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));                        \
+      raised = true;                                                                                               \
+    }                                                                                                              \
+    hipLaunchKernelGGL((window_attn_mfma_kernel<HPW, DKV, VTV, MAXT>), grid, dim3(nthr), lds, st, q, kc, vc, bt,   \
+                       max_pages, cu_q, ctx_len, mix, gate, gate_stride, out, H, G, scale, softcap, slope_exp,     \
+                       window, sink);                                                                              \
+  } while (0)
+  if (D == 64 && V == 64) MFMA_CASE(2, 4);
+  else if (D == 64 && V == 128) MFMA_CASE(2, 8);
+  else if (D == 128 && V == 64) MFMA_CASE(4, 4);
+  else MFMA_CASE(4, 8);
+#undef MFMA_CASE
+  return (int)hipGetLastError();
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) window_attn_combine_kernel(const float* __restrict__ part_acc,
                                                                    const float* __restrict__ part_ml,
+                                                                   const T* __restrict__ gate, int64_t gate_stride,
                                                                    T* __restrict__ out, int H, int V, int nsplit) {
   const size_t tok = blockIdx.x;
   for (int o = threadIdx.x; o < H * V; o += 256) {
@@ -235,7 +463,9 @@ __global__ void __launch_bounds__(256) window_attn_combine_kernel(const float* _
       num += w * part_acc[((tok * nsplit + s) * H + h) * V + v];
       den += w * part_ml[((tok * nsplit + s) * H + h) * 2 + 1];
     }
-    stf<T>(out, (tok * H + h) * V + v, den > 0.f ? num / den : 0.f);
+    float val = den > 0.f ? num / den : 0.f;
+    if (gate) val /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + h));
+    stf<T>(out, (tok * H + h) * V + v, val);
   }
 }
 
@@ -268,12 +498,25 @@ extern "C" int areal_window_attn_tile(int H, int G, int D, int V, int want) {
 // B rows; row b's queries are tokens cu_q[b] .. cu_q[b+1] of q [T, H, D]; max_q = longest row. nsplit > 1 needs
 // part_acc [T, nsplit, H, V] and part_ml [T, nsplit, H, 2] (fp32) and is meant for single-query rows.
 extern "C" int areal_window_attn(const void* q, const void* kcache, const void* vcache, const int* block_tables,
-                                 int max_pages, const int* cu_q, const int* ctx_len, const void* mix, void* out,
-                                 float* part_acc, float* part_ml, int B, int max_q, int T, int H, int G, int D, int V,
+                                 int max_pages, const int* cu_q, const int* ctx_len, const void* mix, const void* gate,
+                                 int64_t gate_stride, void* out, float* part_acc, float* part_ml, int B, int max_q, int T, int H, int G, int D, int V,
                                  int bq, float scale, float softcap, float slope_exp, int window, int sink, int nsplit,
-                                 int dt, hipStream_t st) {
+                                 int dt, int matrix_cores, hipStream_t st) {
   if (B == 0 || T == 0) return 0;
   if (G <= 0 || H % G != 0 || bq <= 0 || nsplit < 1) return -1;
+  if (matrix_cores && dt == 0 && nsplit == 1 && max_q > 1 && mfma_usable(H, G, D, V)) {
+    const int hpw = mfma_heads_per_wave(H), nthr = 64 * (H / hpw);
+    const dim3 mgrid((max_q + 15) / 16, B, 1);
+    const size_t mlds = mfma_lds_bytes(G, D, V);
+#define MFMA_ARGS                                                                                                  \
+  mgrid, nthr, mlds, st, (const bf16_t*)q, (const bf16_t*)kcache, (const bf16_t*)vcache, block_tables, max_pages,   \
+      cu_q, ctx_len, (const bf16_t*)mix, (const bf16_t*)gate, gate_stride, (bf16_t*)out, H, G, D, V, scale, softcap, \
+      slope_exp, window, sink
+    if (hpw == 4) return launch_mfma<4, 256>(MFMA_ARGS);
+    if (hpw == 2) return launch_mfma<2, 512>(MFMA_ARGS);
+    return launch_mfma<1, 512>(MFMA_ARGS);
+#undef MFMA_ARGS
+  }
   AttnShape sh{H, G, D, V, bq};
   const size_t lds = sh.floats() * sizeof(float);
   if (lds > 160 * 1024) return -2;
@@ -288,11 +531,11 @@ extern "C" int areal_window_attn(const void* q, const void* kcache, const void* 
       allowed = 160 * 1024;                                                                                          \
     }                                                                                                                \
     hipLaunchKernelGGL(window_attn_kernel<TT>, grid, dim3(256), lds, st, (const TT*)q, (const TT*)kcache,            \
-                       (const TT*)vcache, block_tables, max_pages, cu_q, ctx_len, (const TT*)mix, (TT*)out, part_acc, \
-                       part_ml, sh, scale, softcap, slope_exp, window, sink, nsplit);                                \
+                       (const TT*)vcache, block_tables, max_pages, cu_q, ctx_len, (const TT*)mix, (const TT*)gate,   \
+                       gate_stride, (TT*)out, part_acc, part_ml, sh, scale, softcap, slope_exp, window, sink, nsplit); \
     if (nsplit > 1)                                                                                                  \
-      hipLaunchKernelGGL(window_attn_combine_kernel<TT>, dim3(T), dim3(256), 0, st, part_acc, part_ml, (TT*)out, H, \
-                         V, nsplit);                                                                                 \
+      hipLaunchKernelGGL(window_attn_combine_kernel<TT>, dim3(T), dim3(256), 0, st, part_acc, part_ml,              \
+                         (const TT*)gate, gate_stride, (TT*)out, H, V, nsplit);                                      \
   } while (0)
   if (dt == 0) LAUNCH(bf16_t);
   else LAUNCH(float);

@@ -68,7 +68,10 @@ def _attention_reference(qn, kn, v, scale, softcap, talk, window):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,V,window", [(4, 2, 16, 24, 37), (3, 3, 8, 8, 32), (6, 1, 40, 16, 5), (2, 2, 64, 64, 0)])
+@pytest.mark.parametrize("H,G,D,V,window", [(4, 2, 16, 24, 37), (3, 3, 8, 8, 32), (6, 1, 40, 16, 5), (2, 2, 64, 64, 0),
+                                            # head sizes the matrix-core kernel takes (bf16 rows of several queries)
+                                            (4, 2, 64, 64, 37), (16, 4, 128, 128, 70), (8, 8, 128, 64, 33),
+                                            (2, 1, 64, 128, 0), (6, 2, 64, 64, 40), (12, 4, 64, 64, 45)])
 def test_window_attention_edges_pages_portions_and_splits(device, dtype, H, G, D, V, window):
     """A key that dominates its query's scores sits just inside and just outside the window, on both sides of page
     borders and at position 0; whole prompt, portions down to two tokens and split decoding must all agree."""
@@ -86,7 +89,7 @@ def test_window_attention_edges_pages_portions_and_splits(device, dtype, H, G, D
     qw = 1 + 0.2 * torch.randn(D, generator=g)
     kw = 1 + 0.2 * torch.randn(D, generator=g)
     talk = torch.eye(H) + 0.2 * torch.randn(H, H, generator=g)
-    proj = torch.cat([q.reshape(n, -1), k.reshape(n, -1), v.reshape(n, -1), torch.randn(n, 3, generator=g)], 1).to(dtype)
+    proj = torch.cat([q.reshape(n, -1), k.reshape(n, -1), v.reshape(n, -1), torch.randn(n, H, generator=g)], 1).to(dtype)
     qw, kw, talk = qw.to(dtype), kw.to(dtype), talk.to(dtype)
     p64 = proj.to(F64)
     qn = O.unit_rms(p64[:, :H * D].view(n, H, D), eps) * qw.to(F64)
@@ -95,13 +98,14 @@ def test_window_attention_edges_pages_portions_and_splits(device, dtype, H, G, D
         qn, kn = qn.to(dtype).to(F64), kn.to(dtype).to(F64)
     want = _attention_reference(qn, kn, p64[:, (H + G) * D:(H + G) * D + G * V].view(n, G, V), scale, softcap,
                                 talk.to(F64), window)
+    want = want * torch.sigmoid(p64[:, -H:]).unsqueeze(-1)  # one gate per head and token
     shape = wattn.ScoreShape(scale=scale, softcap=softcap, slope_exp=8.0, window=window, sink=True)
     pages = [7, 2, 9, 4, 1]  # scattered, out of order
     bt = torch.tensor([pages], dtype=torch.int32, device=device)
     slots = torch.tensor([pages[t // 32] * 32 + t % 32 for t in range(n)], dtype=torch.int64, device=device)
     pj, qwd, kwd, tk = proj.to(device), qw.to(device), kw.to(device), talk.to(device)
 
-    def run(portions, nsplit=1):
+    def run(portions, nsplit=1, matrix_cores=True):
         kc, vc = wattn.alloc_window_cache(12, G, D, V, dtype, device)
         kc.fill_(float("nan") if dtype == torch.float32 else 1e4)  # stale pages must never leak into a result
         vc.fill_(1e4)
@@ -111,7 +115,8 @@ def test_window_attention_edges_pages_portions_and_splits(device, dtype, H, G, D
             cu = torch.tensor([0, c], dtype=torch.int32, device=device)
             ctx = torch.tensor([at + c], dtype=torch.int32, device=device)
             outs.append(wattn.window_attention(qq, kc, vc, bt, cu, ctx, c, shape, tk,
-                                               nsplit=nsplit if c == 1 else 1))
+                                               nsplit=nsplit if c == 1 else 1, gate=pj[at:at + c, -H:],
+                                               matrix_cores=matrix_cores))
             at += c
         return torch.cat(outs).float().cpu()
 
@@ -120,6 +125,8 @@ def test_window_attention_edges_pages_portions_and_splits(device, dtype, H, G, D
     cut = run([3, 64, 2, 50, 29, 2])
     assert rel_err(cut.reshape(n, -1), want.reshape(n, -1)) < tol(dtype)
     assert rel_err(cut.reshape(n, -1), whole.reshape(n, -1)) < 1e-5 + (1e-2 if dtype == torch.bfloat16 else 0)
+    plain = run([3, 64, 2, 50, 29, 2], matrix_cores=False)  # the kernel for every shape and type
+    assert rel_err(plain.reshape(n, -1), want.reshape(n, -1)) < tol(dtype)
     for nsplit in (1, 3):
         dec = run([100] + [1] * 50, nsplit=nsplit)
         assert rel_err(dec.reshape(n, -1), want.reshape(n, -1)) < tol(dtype)
@@ -332,6 +339,7 @@ SHAPES = [
            vocab=67, alpha=0.9),
     config([attn_layer(4, 2, 16, 24, 0)], width=24),  # no window: every earlier token is seen
     config([mlstm_layer(2, 72, 80, cap=12.0)], width=56, alpha=3.0, eps=1e-3),
+    config([attn_layer(4, 2, 64, 64, 37), mlstm_layer(2, 64, 64), attn_layer(8, 2, 64, 128, 50, ff=0)], width=64),
 ]
 
 
@@ -382,6 +390,31 @@ def test_greedy_generation_through_the_engine(device, dtype):
                 same = sum(1 for a, b in zip(r.output_tokens, want) if a == b)
                 assert r.output_tokens[:4] == want[:4] and same >= 6
         assert eng.sched.num_free_state_slots() == 3
+    finally:
+        eng.destroy()
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_served_from_a_checkpoint_directory(device, tmp_path):
+    """The framework's own path from a directory with config.json and model.safetensors: the model class is chosen by
+    the configuration, the weights come through the engine's loader."""
+    from areal_vllm_amd.models import build_model
+
+    cfg_dict = config([mlstm_layer(2, 8, 16), attn_layer(4, 1, 8, 16, 9, ff=0)], width=32, vocab=53)
+    m = build_model(ModelConfig.from_hf_dict(cfg_dict), dtype=torch.bfloat16)
+    m.flatten()
+    m.init_weights(seed=9)
+    m.save_checkpoint(str(tmp_path))
+    w = {k: v.float() for k, v in m.checkpoint_tensors().items()}
+    srv = InferenceServerConfig(model_path=str(tmp_path), dtype="float32", context_length=128, max_running_requests=2,
+                                num_continuous_decode_steps=2)
+    eng = NativeInferenceEngine(srv, device=torch.device(device), num_pages=12)
+    eng.initialize()
+    try:
+        prompts = [tokens_of(n, 53, 70 + n) for n in (5, 33, 17)]
+        res = eng.generate_blocking(prompts, max_new_tokens=7, greedy=True)
+        for p, r in zip(prompts, res):
+            assert r.output_tokens == O.greedy(p, 7, w, cfg_dict)
     finally:
         eng.destroy()
 
