@@ -55,10 +55,12 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, ig: torch
     T = proj.shape[0]
     NH, D, V = state.S.shape[1], state.S.shape[2], state.S.shape[3]
     B = cu_q.numel() - 1
-    hbuf = torch.zeros(T, NH, V, dtype=torch.float32, device=proj.device)
-    nq = torch.zeros(T, NH, dtype=torch.float32, device=proj.device)
-    mt = torch.zeros(T, NH, dtype=torch.float32, device=proj.device)
-    if L.use_hip(proj):
+    hip = L.use_hip(proj)
+    new = torch.empty if hip else torch.zeros  # the kernel writes every element (zeros for skipped rows)
+    hbuf = new(T, NH, V, dtype=torch.float32, device=proj.device)
+    nq = new(T, NH, dtype=torch.float32, device=proj.device)
+    mt = new(T, NH, dtype=torch.float32, device=proj.device)
+    if hip:
         assert proj.stride(1) == 1 and cu_q.dtype == torch.int32 and first_pos.dtype == torch.int32
         assert state_slots.dtype == torch.int32 and ig.is_contiguous() and fg.is_contiguous()
         if D > 256:

@@ -67,10 +67,11 @@ def qk_norm_cache_write(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_
 
 
 def decode_splits(batch: int, window: int, max_context: int) -> int:
-    """Key-range splits of a decode launch: enough workgroups to occupy the device, at least a few pages each."""
+    """Key-range splits of a decode launch: about two workgroups per compute unit, down to one page each (a
+    workgroup walks its pages one after the other, so short ranges are what makes a decode step short)."""
     span = max_context if window <= 0 else min(window + PAGE_SIZE, max_context)
     pages = max(1, (span + PAGE_SIZE - 1) // PAGE_SIZE)
-    return int(max(1, min(256 // max(1, batch), pages // 4, 32)))
+    return int(max(1, min(512 // max(1, batch), pages, 32)))
 
 
 def window_attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_tables: torch.Tensor,

@@ -11,9 +11,9 @@
 //
 // `mlstm_gates`: i = cap tanh((W_i x + b_i) / cap), f = logsigmoid(cap tanh((W_f x + b_f) / cap)) with fp32
 // accumulation of the dot products (the gates enter exponentials of running sums, so they never pass through bf16).
-// `mlstm_scan`: one wave per (row, head, 64 value columns). Lane c keeps column c of S in registers (D values),
-// the wave keeps n spread over its lanes; keys and queries of a few tokens at a time are staged in LDS as fp32. It
-// writes the unnormalised read-out S_t^T q_t, n_t . q_t and m_t; `mlstm_out` divides, applies the per-head RMS norm,
+// `mlstm_scan`: one workgroup of four waves per (row, head, 64 value columns); every wave keeps a quarter of the
+// rows of S (lane c: column c) and of n in registers; keys and queries of a few tokens at a time are staged in LDS as
+// fp32. It writes the unnormalised read-out S_t^T q_t, n_t . q_t and m_t; `mlstm_out` divides, applies the per-head RMS norm,
 // the weight and the sigmoid output gate.
 #include "common.hpp"
 
@@ -26,20 +26,31 @@ template <typename T> DEVINL void stf(T* p, size_t i, float v);
 template <> DEVINL void stf<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f2bf(v); }
 template <> DEVINL void stf<float>(float* p, size_t i, float v) { p[i] = v; }
 
-// w [2 * NH, W]: rows of the input gate's heads, then of the forget gate's; b [2 * NH]
-template <typename T>
+// w [2 * NH, W]: rows of the input gate's heads, then of the forget gate's; b [2 * NH]. A workgroup takes GT tokens
+// and four gate rows (one a wave), so a weight row is read once per GT tokens; decode batches run GT = 1 for the
+// sake of more workgroups.
+template <typename T, int GT>
 __global__ void __launch_bounds__(256) mlstm_gates_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                            const T* __restrict__ bias, float* __restrict__ ig,
-                                                           float* __restrict__ fg, int W, int NH, float cap) {
-  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const T* xr = x + (size_t)t * W;
-  for (int u = wave; u < 2 * NH; u += 4) {
-    const T* wr = w + (size_t)u * W;
-    float s = 0.f;
-    for (int i = lane; i < W; i += 64) s += ldf<T>(xr, i) * ldf<T>(wr, i);
-    s = wave_sum(s);
-    if (lane == 0) {
-      float z = s + (bias ? ldf<T>(bias, u) : 0.f);
+                                                           float* __restrict__ fg, int Ttok, int W, int NH, float cap) {
+  const int t0 = blockIdx.x * GT, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int u = blockIdx.y * 4 + wave;
+  if (u >= 2 * NH) return;
+  const T* wr = w + (size_t)u * W;
+  float s[GT];
+#pragma unroll
+  for (int tt = 0; tt < GT; ++tt) s[tt] = 0.f;
+  for (int i = lane; i < W; i += 64) {
+    const float wv = ldf<T>(wr, i);
+#pragma unroll
+    for (int tt = 0; tt < GT; ++tt) s[tt] += ldf<T>(x, (size_t)min(t0 + tt, Ttok - 1) * W + i) * wv;
+  }
+#pragma unroll
+  for (int tt = 0; tt < GT; ++tt) {
+    const float tot = wave_sum(s[tt]);
+    const int t = t0 + tt;
+    if (lane == 0 && t < Ttok) {
+      float z = tot + (bias ? ldf<T>(bias, u) : 0.f);
       if (cap > 0.f) z = cap * tanhf(z / cap);
       if (u < NH) ig[(size_t)t * NH + u] = z;
       else fg[(size_t)t * NH + (u - NH)] = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));  // log sigmoid
@@ -48,92 +59,117 @@ __global__ void __launch_bounds__(256) mlstm_gates_kernel(const T* __restrict__ 
 }
 
 constexpr int TC = 8;  // tokens staged per round
+constexpr int RW = 4;  // waves of a workgroup: each keeps a quarter of the state's rows
 
+// One workgroup per (row, head, 64 value columns). Wave r keeps rows r DQ .. r DQ + DQ - 1 of S (lane c: column c) and
+// of n (lane i: row i of its quarter) in registers. Per round of TC tokens every wave forms its partial read-outs,
+// the partials meet in LDS and wave r finishes tokens r and r + RW.
 template <typename T, int DP>
-__global__ void __launch_bounds__(64) mlstm_scan_kernel(
+__global__ void __launch_bounds__(64 * RW) mlstm_scan_kernel(
     const T* __restrict__ proj, int64_t row_stride, int q_off, int k_off, int v_off, const float* __restrict__ ig,
     const float* __restrict__ fg, const int* __restrict__ cu_q, const int* __restrict__ first_pos,
     const int* __restrict__ state_slots, float* __restrict__ S, float* __restrict__ N, float* __restrict__ M,
     float* __restrict__ hbuf, float* __restrict__ nq, float* __restrict__ mt, int NH, int D, int V) {
-  constexpr int NN = (DP + 63) / 64;
+  constexpr int DQ = DP / RW;
   __shared__ float kq[TC][2][DP];
-  const int b = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x;
+  __shared__ float hpart[RW][TC][64];
+  __shared__ float npart[RW][TC];
+  const int b = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, lane = tid & 63, r = tid >> 6;
   const int col = blockIdx.z * 64 + lane;
   const bool has = col < V;
   const int slot = state_slots[b];
   const int t_lo = cu_q[b], t_hi = cu_q[b + 1];
-  if (slot < 0 || t_hi <= t_lo) return;
+  if (slot < 0) {  // a retired row: its outputs are defined (zero), no slot is touched
+    if (r == 0)
+      for (int t = t_lo; t < t_hi; ++t) {
+        if (has) hbuf[((size_t)t * NH + hd) * V + col] = 0.f;
+        if (blockIdx.z == 0 && lane == 0) nq[(size_t)t * NH + hd] = mt[(size_t)t * NH + hd] = 0.f;
+      }
+    return;
+  }
+  if (t_hi <= t_lo) return;
   const bool fresh = first_pos[b] == 0;
   const size_t sbase = ((size_t)slot * NH + hd) * D;
-  float s[DP], nn[NN];
+  const int d0 = r * DQ;
+  float s[DQ];
 #pragma unroll
-  for (int d = 0; d < DP; ++d) s[d] = (!fresh && has && d < D) ? S[(sbase + d) * V + col] : 0.f;
-#pragma unroll
-  for (int i = 0; i < NN; ++i) {
-    const int d = lane + 64 * i;
-    nn[i] = (!fresh && d < D) ? N[sbase + d] : 0.f;
-  }
+  for (int d = 0; d < DQ; ++d) s[d] = (!fresh && has && d0 + d < D) ? S[(sbase + d0 + d) * V + col] : 0.f;
+  const int nd = d0 + lane;  // the row of n this lane keeps
+  const bool nlive = lane < DQ && nd < D;
+  float nn = (!fresh && nlive) ? N[sbase + nd] : 0.f;
   float m = fresh ? 0.f : M[(size_t)slot * NH + hd];
   const float qscale = 1.f / sqrtf((float)D);
   for (int tb = t_lo; tb < t_hi; tb += TC) {
     const int nt = min(TC, t_hi - tb);
-    __syncthreads();
-    for (int i = lane; i < nt * DP; i += 64) {
+    __syncthreads();  // the round before is finished with kq and the partials
+    for (int i = tid; i < nt * DP; i += 64 * RW) {
       const int d = i % DP, tt = i / DP;
       const T* row = proj + (size_t)(tb + tt) * row_stride;
       kq[tt][0][d] = d < D ? ldf<T>(row, k_off + hd * D + d) : 0.f;
       kq[tt][1][d] = d < D ? ldf<T>(row, q_off + hd * D + d) * qscale : 0.f;
     }
-    float vv[TC];
-#pragma unroll
-    for (int tt = 0; tt < TC; ++tt)
-      vv[tt] = (tt < nt && has) ? ldf<T>(proj + (size_t)(tb + tt) * row_stride, v_off + hd * V + col) : 0.f;
-    __syncthreads();
+    float vv[TC], fgr[TC], igr[TC];  // loaded ahead: nothing inside the recurrence waits for memory
 #pragma unroll
     for (int tt = 0; tt < TC; ++tt) {
+      vv[tt] = (tt < nt && has) ? ldf<T>(proj + (size_t)(tb + tt) * row_stride, v_off + hd * V + col) : 0.f;
+      fgr[tt] = tt < nt ? fg[(size_t)(tb + tt) * NH + hd] : 0.f;
+      igr[tt] = tt < nt ? ig[(size_t)(tb + tt) * NH + hd] : 0.f;
+    }
+    __syncthreads();
+    float mloc[TC];
+#pragma unroll
+    for (int tt = 0; tt < TC; ++tt) {
+      mloc[tt] = m;
       if (tt < nt) {
-        const size_t th = (size_t)(tb + tt) * NH + hd;
-        const float f = fg[th], ii = ig[th];
+        const float f = fgr[tt], ii = igr[tt];
         const float m2 = fmaxf(f + m, ii);
         const float a = expf(f + m - m2), bb = expf(ii - m2);
         m = m2;
+        mloc[tt] = m;
         const float bv = bb * vv[tt];
         float hacc = 0.f;
 #pragma unroll
-        for (int d = 0; d < DP; ++d) {
-          s[d] = a * s[d] + bv * kq[tt][0][d];
-          hacc += s[d] * kq[tt][1][d];
+        for (int d = 0; d < DQ; ++d) {
+          s[d] = a * s[d] + bv * kq[tt][0][d0 + d];
+          hacc += s[d] * kq[tt][1][d0 + d];
         }
         float part = 0.f;
-#pragma unroll
-        for (int i = 0; i < NN; ++i) {
-          const int d = lane + 64 * i;
-          if (d < DP) {
-            nn[i] = a * nn[i] + bb * kq[tt][0][d];
-            part += nn[i] * kq[tt][1][d];
-          }
+        if (lane < DQ) {
+          nn = a * nn + bb * kq[tt][0][nd];
+          part = nn * kq[tt][1][nd];
         }
         part = wave_sum(part);
-        if (has) hbuf[th * V + col] = hacc;
+        hpart[r][tt][lane] = hacc;
+        if (lane == 0) npart[r][tt] = part;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < TC; ++tt) {
+      if (tt < nt && (tt % RW) == r) {
+        const size_t th = (size_t)(tb + tt) * NH + hd;
+        float hsum = 0.f, nsum = 0.f;
+#pragma unroll
+        for (int w = 0; w < RW; ++w) {
+          hsum += hpart[w][tt][lane];
+          nsum += npart[w][tt];
+        }
+        if (has) hbuf[th * V + col] = hsum;
         if (blockIdx.z == 0 && lane == 0) {
-          nq[th] = part;
-          mt[th] = m;
+          nq[th] = nsum;
+          mt[th] = mloc[tt];
         }
       }
     }
   }
   if (has) {
 #pragma unroll
-    for (int d = 0; d < DP; ++d)
-      if (d < D) S[(sbase + d) * V + col] = s[d];
+    for (int d = 0; d < DQ; ++d)
+      if (d0 + d < D) S[(sbase + d0 + d) * V + col] = s[d];
   }
   if (blockIdx.z == 0) {
-#pragma unroll
-    for (int i = 0; i < NN; ++i) {
-      const int d = lane + 64 * i;
-      if (d < D) N[sbase + d] = nn[i];
-    }
-    if (lane == 0) M[(size_t)slot * NH + hd] = m;
+    if (nlive) N[sbase + nd] = nn;
+    if (tid == 0) M[(size_t)slot * NH + hd] = m;
   }
 }
 
@@ -168,12 +204,18 @@ __global__ void __launch_bounds__(256) mlstm_out_kernel(const float* __restrict_
 extern "C" int areal_mlstm_gates(const void* x, const void* w, const void* bias, float* ig, float* fg, int T, int W,
                                  int NH, float cap, int dt, hipStream_t st) {
   if (T == 0) return 0;
-  if (dt == 0)
-    hipLaunchKernelGGL(mlstm_gates_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)w,
-                       (const bf16_t*)bias, ig, fg, W, NH, cap);
-  else
-    hipLaunchKernelGGL(mlstm_gates_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)x, (const float*)w,
-                       (const float*)bias, ig, fg, W, NH, cap);
+  const int rows = (2 * NH + 3) / 4;
+#define LAUNCH(TT, GTV)                                                                                           \
+  hipLaunchKernelGGL((mlstm_gates_kernel<TT, GTV>), dim3((T + GTV - 1) / GTV, rows), dim3(256), 0, st, (const TT*)x, \
+                     (const TT*)w, (const TT*)bias, ig, fg, T, W, NH, cap)
+  if (dt == 0) {
+    if (T < 512) LAUNCH(bf16_t, 1);
+    else LAUNCH(bf16_t, 8);
+  } else {
+    if (T < 512) LAUNCH(float, 1);
+    else LAUNCH(float, 8);
+  }
+#undef LAUNCH
   return (int)hipGetLastError();
 }
 
@@ -187,7 +229,7 @@ extern "C" int areal_mlstm_scan(const void* proj, int64_t row_stride, int q_off,
   if (D > 256 || D <= 0 || V <= 0) return -1;
   const dim3 grid(B, NH, (V + 63) / 64);
 #define LAUNCH(TT, DPV)                                                                                          \
-  hipLaunchKernelGGL((mlstm_scan_kernel<TT, DPV>), grid, dim3(64), 0, st, (const TT*)proj, row_stride, q_off,    \
+  hipLaunchKernelGGL((mlstm_scan_kernel<TT, DPV>), grid, dim3(64 * RW), 0, st, (const TT*)proj, row_stride, q_off,    \
                      k_off, v_off, ig, fg, cu_q, first_pos, state_slots, S, N, M, hbuf, nq, mt, NH, D, V)
 #define PICK(TT)                 \
   do {                           \

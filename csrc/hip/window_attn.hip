@@ -137,7 +137,16 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
     for (int c = 0; c < G; ++c) {
       __syncthreads();  // Kt free (and, first time round, the tile set-up visible)
       const T* kp = kcache + ((page * G + c) * PAGE) * D;
-      for (int i = tid; i < PAGE * D; i += 256) Kt[(i / D) * (D + 1) + i % D] = ldf<T>(kp, i);
+      if (sizeof(T) == 2 && D % 8 == 0) {  // 16-byte loads
+        for (int i = tid; i < PAGE * D / 8; i += 256) {
+          const bf16x8 x = ld8(reinterpret_cast<const bf16_t*>(kp) + 8 * i);
+          float* dst = Kt + (8 * i / D) * (D + 1) + (8 * i) % D;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) dst[e] = bf2f(x[e]);
+        }
+      } else {
+        for (int i = tid; i < PAGE * D; i += 256) Kt[(i / D) * (D + 1) + i % D] = ldf<T>(kp, i);
+      }
       __syncthreads();
       for (int e = tid; e < rep * BQ * PAGE; e += 256) {
         const int kj = e % PAGE, r = e / PAGE, qi = r % BQ, g = c * rep + r / BQ;
@@ -190,7 +199,16 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
     for (int c = 0; c < G; ++c) {
       __syncthreads();  // Vt free; weights and corr visible
       const T* vp = vcache + ((page * G + c) * PAGE) * V;
-      for (int i = tid; i < PAGE * V; i += 256) Vt[i] = (jb + i / V < j_hi) ? ldf<T>(vp, i) : 0.f;
+      if (sizeof(T) == 2 && V % 8 == 0) {
+        for (int i = tid; i < PAGE * V / 8; i += 256) {
+          const bf16x8 x = ld8(reinterpret_cast<const bf16_t*>(vp) + 8 * i);
+          const bool live = jb + (8 * i) / V < j_hi;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) Vt[8 * i + e] = live ? bf2f(x[e]) : 0.f;
+        }
+      } else {
+        for (int i = tid; i < PAGE * V; i += 256) Vt[i] = (jb + i / V < j_hi) ? ldf<T>(vp, i) : 0.f;
+      }
       __syncthreads();
       for (int o = tid; o < rep * BQ * V; o += 256) {
         const int v = o % V, rr = o / V;
