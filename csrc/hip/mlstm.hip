@@ -99,22 +99,47 @@ __global__ void __launch_bounds__(64 * RW) mlstm_scan_kernel(
   float nn = (!fresh && nlive) ? N[sbase + nd] : 0.f;
   float m = fresh ? 0.f : M[(size_t)slot * NH + hd];
   const float qscale = 1.f / sqrtf((float)D);
+  // operands of a round are fetched into registers one round ahead, so the loads' latency runs under the
+  // recurrence of the round before
+  constexpr int KQN = (TC * DP + 64 * RW - 1) / (64 * RW);
+  float pk[KQN], pq[KQN], pv[TC], pf[TC], pi[TC];
+  auto fetch = [&](int tb) {
+    const int nt = min(TC, t_hi - tb);
+#pragma unroll
+    for (int j = 0; j < KQN; ++j) {
+      const int i = tid + j * 64 * RW, d = i % DP, tt = i / DP;
+      const bool live = tt < nt && d < D;
+      const T* row = proj + (size_t)(tb + min(tt, nt - 1)) * row_stride;
+      pk[j] = live ? ldf<T>(row, k_off + hd * D + d) : 0.f;
+      pq[j] = live ? ldf<T>(row, q_off + hd * D + d) * qscale : 0.f;
+    }
+#pragma unroll
+    for (int tt = 0; tt < TC; ++tt) {
+      pv[tt] = (tt < nt && has) ? ldf<T>(proj + (size_t)(tb + tt) * row_stride, v_off + hd * V + col) : 0.f;
+      pf[tt] = tt < nt ? fg[(size_t)(tb + tt) * NH + hd] : 0.f;
+      pi[tt] = tt < nt ? ig[(size_t)(tb + tt) * NH + hd] : 0.f;
+    }
+  };
+  fetch(t_lo);
   for (int tb = t_lo; tb < t_hi; tb += TC) {
     const int nt = min(TC, t_hi - tb);
     __syncthreads();  // the round before is finished with kq and the partials
-    for (int i = tid; i < nt * DP; i += 64 * RW) {
-      const int d = i % DP, tt = i / DP;
-      const T* row = proj + (size_t)(tb + tt) * row_stride;
-      kq[tt][0][d] = d < D ? ldf<T>(row, k_off + hd * D + d) : 0.f;
-      kq[tt][1][d] = d < D ? ldf<T>(row, q_off + hd * D + d) * qscale : 0.f;
+#pragma unroll
+    for (int j = 0; j < KQN; ++j) {
+      const int i = tid + j * 64 * RW;
+      if (i < TC * DP) {
+        kq[i / DP][0][i % DP] = pk[j];
+        kq[i / DP][1][i % DP] = pq[j];
+      }
     }
-    float vv[TC], fgr[TC], igr[TC];  // loaded ahead: nothing inside the recurrence waits for memory
+    float vv[TC], fgr[TC], igr[TC];
 #pragma unroll
     for (int tt = 0; tt < TC; ++tt) {
-      vv[tt] = (tt < nt && has) ? ldf<T>(proj + (size_t)(tb + tt) * row_stride, v_off + hd * V + col) : 0.f;
-      fgr[tt] = tt < nt ? fg[(size_t)(tb + tt) * NH + hd] : 0.f;
-      igr[tt] = tt < nt ? ig[(size_t)(tb + tt) * NH + hd] : 0.f;
+      vv[tt] = pv[tt];
+      fgr[tt] = pf[tt];
+      igr[tt] = pi[tt];
     }
+    if (tb + TC < t_hi) fetch(tb + TC);
     __syncthreads();
     float mloc[TC];
 #pragma unroll

@@ -465,25 +465,26 @@ int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q
   return (int)hipGetLastError();
 }
 
+// one workgroup per (token, head): thread v merges the splits' partial sums of value column v
 template <typename T>
-__global__ void __launch_bounds__(256) window_attn_combine_kernel(const float* __restrict__ part_acc,
+__global__ void __launch_bounds__(128) window_attn_combine_kernel(const float* __restrict__ part_acc,
                                                                    const float* __restrict__ part_ml,
                                                                    const T* __restrict__ gate, int64_t gate_stride,
                                                                    T* __restrict__ out, int H, int V, int nsplit) {
   const size_t tok = blockIdx.x;
-  for (int o = threadIdx.x; o < H * V; o += 256) {
-    const int h = o / V, v = o % V;
-    float M = -1e30f;
-    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[((tok * nsplit + s) * H + h) * 2]);
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float w = expf(part_ml[((tok * nsplit + s) * H + h) * 2] - M);
-      num += w * part_acc[((tok * nsplit + s) * H + h) * V + v];
-      den += w * part_ml[((tok * nsplit + s) * H + h) * 2 + 1];
-    }
-    float val = den > 0.f ? num / den : 0.f;
-    if (gate) val /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + h));
-    stf<T>(out, (tok * H + h) * V + v, val);
+  const int h = blockIdx.y;
+  float M = -1e30f;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[((tok * nsplit + s) * H + h) * 2]);
+  float den = 0.f;
+  for (int s = 0; s < nsplit; ++s)
+    den += expf(part_ml[((tok * nsplit + s) * H + h) * 2] - M) * part_ml[((tok * nsplit + s) * H + h) * 2 + 1];
+  float f = den > 0.f ? 1.f / den : 0.f;
+  if (gate) f /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + h));
+  for (int v = threadIdx.x; v < V; v += 128) {
+    float num = 0.f;
+    for (int s = 0; s < nsplit; ++s)
+      num += expf(part_ml[((tok * nsplit + s) * H + h) * 2] - M) * part_acc[((tok * nsplit + s) * H + h) * V + v];
+    stf<T>(out, (tok * H + h) * V + v, num * f);
   }
 }
 
@@ -552,7 +553,7 @@ extern "C" int areal_window_attn(const void* q, const void* kcache, const void* 
                        (const TT*)vcache, block_tables, max_pages, cu_q, ctx_len, (const TT*)mix, (const TT*)gate,   \
                        gate_stride, (TT*)out, part_acc, part_ml, sh, scale, softcap, slope_exp, window, sink, nsplit); \
     if (nsplit > 1)                                                                                                  \
-      hipLaunchKernelGGL(window_attn_combine_kernel<TT>, dim3(T), dim3(256), 0, st, part_acc, part_ml,              \
+      hipLaunchKernelGGL(window_attn_combine_kernel<TT>, dim3(T, H), dim3(128), 0, st, part_acc, part_ml,           \
                          (const TT*)gate, gate_stride, (TT*)out, H, V, nsplit);                                      \
   } while (0)
   if (dt == 0) LAUNCH(bf16_t);
