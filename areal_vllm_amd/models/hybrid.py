@@ -99,20 +99,6 @@ def kuzanex_config_from_dir(path: str) -> HybridConfig:
     return cfg
 
 
-DECODE_GEMM_MAX_ROWS = 256
-
-
-def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x @ w.T (+ bias). Few bf16 rows on the GPU (a decode batch) stream the weight through the framework's decode
-    GEMM (``ops/decode_gemm.py``) where its tile shapes fit, everything else through the library."""
-    if (x.is_cuda and x.dtype == torch.bfloat16 and x.shape[0] <= DECODE_GEMM_MAX_ROWS and w.shape[1] % 64 == 0
-            and w.shape[0] % 32 == 0 and x.stride(1) == 1 and w.is_contiguous()):
-        from ..ops import decode_gemm as dg
-
-        return dg.dgemm(x, w, bias, epilogue=dg.EPI_BF16)
-    return F.linear(x, w, bias)
-
-
 class StepTensors:
     """What one batch plan hands to the mixers (all on the device): rows of the packed token batch (`cu_q`, longest
     row `max_q`), each row's context length after the step, cache slot of every token, page tables, position of each
@@ -150,12 +136,12 @@ class WindowAttentionMixer(nn.Module):
         kc, vc = cache
         T = xc.shape[0]
         H, G, D, V = self.H, self.G, self.D, self.V
-        proj = linear(xc, self.proj, self.proj_bias)
+        proj = F.linear(xc, self.proj, self.proj_bias)
         q = wattn.qk_norm_cache_write(proj, self.q_norm, self.k_norm, st.slots, kc, vc, H, self.eps)
         o = wattn.window_attention(q, kc, vc, st.block_tables, st.cu_q, st.ctx_len, st.max_q, self.shape, self.talk,
                                    nsplit=st.nsplit if st.max_q == 1 else 1, workspace=st.workspace,
                                    gate=proj[:, (H + G) * D + G * V:])
-        return linear(o.view(T, H * V), self.o)
+        return F.linear(o.view(T, H * V), self.o)
 
 
 class MLSTMMixer(nn.Module):
@@ -176,12 +162,12 @@ class MLSTMMixer(nn.Module):
 
     def step(self, xc: torch.Tensor, st: StepTensors, state) -> torch.Tensor:
         H, D, V = self.H, self.D, self.V
-        proj = linear(xc, self.proj)
+        proj = F.linear(xc, self.proj)
         ig, fg = mlstm_ops.mlstm_gates(xc, self.gates, self.gates_bias, H, self.cap)
         hbuf, nq, mt = mlstm_ops.mlstm_scan(proj, 0, H * D, 2 * H * D, ig, fg, st.cu_q, st.first_pos, st.state_slots,
                                             state)
         y = mlstm_ops.mlstm_out(hbuf, nq, mt, proj[:, 2 * H * D + H * V:], self.norm, self.eps)
-        return linear(y, self.o)
+        return F.linear(y, self.o)
 
 
 class XieluMLP(nn.Module):
@@ -194,7 +180,7 @@ class XieluMLP(nn.Module):
         self.act = nn.Parameter(torch.zeros(2, dtype=dtype, device=device))
 
     def forward(self, xc: torch.Tensor) -> torch.Tensor:
-        return linear(post_norm.xielu(linear(xc, self.up, self.up_bias), self.act), self.down, self.down_bias)
+        return F.linear(post_norm.xielu(F.linear(xc, self.up, self.up_bias), self.act), self.down, self.down_bias)
 
 
 class HybridBlock(nn.Module):
