@@ -165,7 +165,7 @@ class MLSTMMixer(nn.Module):
         proj = F.linear(xc, self.proj)
         ig, fg = mlstm_ops.mlstm_gates(xc, self.gates, self.gates_bias, H, self.cap)
         hbuf, nq, mt = mlstm_ops.mlstm_scan(proj, 0, H * D, 2 * H * D, ig, fg, st.cu_q, st.first_pos, st.state_slots,
-                                            state)
+                                            state, max_q=st.max_q)
         y = mlstm_ops.mlstm_out(hbuf, nq, mt, proj[:, 2 * H * D + H * V:], self.norm, self.eps)
         return F.linear(y, self.o)
 

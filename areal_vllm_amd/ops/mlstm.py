@@ -46,12 +46,13 @@ def mlstm_gates(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 
 
 def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, ig: torch.Tensor, fg: torch.Tensor,
-               cu_q: torch.Tensor, first_pos: torch.Tensor, state_slots: torch.Tensor, state: RecurrentState
-               ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+               cu_q: torch.Tensor, first_pos: torch.Tensor, state_slots: torch.Tensor, state: RecurrentState,
+               max_q: int = 1) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Advance the state of every row's slot over the row's tokens. proj [T, *] holds heads x D queries at column
     q_off, heads x D keys at k_off, heads x V values at v_off. first_pos [B] int32: position of each row's first
-    token (0: fresh state); state_slots [B] int32 (negative: the row is skipped). Returns the unnormalised read-out
-    [T, heads, V], n . q [T, heads] and m [T, heads], fp32."""
+    token (0: fresh state); state_slots [B] int32 (negative: the row is skipped). `max_q`: the longest row; from 16
+    tokens on (key size <= 128) the GPU runs the chunk-parallel kernel on the fp32 matrix cores, otherwise the
+    token-by-token one. Returns the unnormalised read-out [T, heads, V], n . q [T, heads] and m [T, heads], fp32."""
     T = proj.shape[0]
     NH, D, V = state.S.shape[1], state.S.shape[2], state.S.shape[3]
     B = cu_q.numel() - 1
@@ -69,7 +70,7 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, ig: torch
             L.ptr(proj), L.c_int64(proj.stride(0)), L.c_int(q_off), L.c_int(k_off), L.c_int(v_off), L.ptr(ig),
             L.ptr(fg), L.ptr(cu_q), L.ptr(first_pos), L.ptr(state_slots), L.ptr(state.S), L.ptr(state.n),
             L.ptr(state.m), L.ptr(hbuf), L.ptr(nq), L.ptr(mt), L.c_int(B), L.c_int(NH), L.c_int(D), L.c_int(V),
-            L.c_int(L.dtype_flag(proj)), L.stream_ptr()), "mlstm_scan")
+            L.c_int(int(max_q)), L.c_int(L.dtype_flag(proj)), L.stream_ptr()), "mlstm_scan")
         return hbuf, nq, mt
     cq, fp, sl = cu_q.tolist(), first_pos.tolist(), state_slots.tolist()
     qs = 1.0 / math.sqrt(D)

@@ -198,6 +198,206 @@ __global__ void __launch_bounds__(64 * RW) mlstm_scan_kernel(
   }
 }
 
+// Chunk-parallel form of the same recurrence for prompt portions (fp32 matrix cores, MFMA 16x16x4). For a chunk of
+// up to 64 tokens of one row, with F_t the running sum of the log forget gates inside the chunk, b_s = i_s - F_s and
+// g_t = max(m_prev, max_{s <= t} b_s)  (so that m_t = F_t + g_t, the stabiliser of the token-by-token form):
+//
+//   read-out_t = exp(m_prev - g_t) S_prev^T q_t + sum_{s <= t} exp(b_s - g_t) (q_t . k_s) v_s        (n . q likewise)
+//   S_new      = exp(m_prev - g_L) S_prev + sum_s exp(b_s - g_L) k_s v_s^T,   m_new = F_L + g_L
+//
+// Every exponent is <= 0. One workgroup (four waves) per (row, head, 64 value columns) walks the row's chunks; the
+// state slice S [D, 64] lives in LDS between them. Wave w owns tokens 16 w .. 16 w + 15 of the chunk for q k^T and the
+// read-out, and row blocks w, w + 4, .. of S for the update. Key size up to 128.
+constexpr int CL = 64;
+template <typename T, int DP>
+__global__ void __launch_bounds__(256) mlstm_chunk_kernel(
+    const T* __restrict__ proj, int64_t row_stride, int q_off, int k_off, int v_off, const float* __restrict__ ig,
+    const float* __restrict__ fg, const int* __restrict__ cu_q, const int* __restrict__ first_pos,
+    const int* __restrict__ state_slots, float* __restrict__ S, float* __restrict__ N, float* __restrict__ M,
+    float* __restrict__ hbuf, float* __restrict__ nq, float* __restrict__ mt, int NH, int D, int V) {
+  constexpr int QS = DP + 4, CS = CL + 4;
+  extern __shared__ float cl[];
+  float* Sst = cl;                 // [DP][CS] state slice
+  float* Qs = Sst + DP * CS;       // [CL][QS] queries / sqrt(D)
+  float* Ks = Qs + CL * QS;        // [CL][QS]
+  float* Vs = Ks + CL * QS;        // [CL][CS] values of this column slice
+  float* Ps = Vs + CL * CS;        // [CL][CS] weighted q.k
+  float* nst = Ps + CL * CS;       // [DP]
+  float* Fs = nst + DP;            // [CL] running log forget
+  float* bs = Fs + CL;             // [CL]
+  float* gs = bs + CL;             // [CL]
+  float* nqs = gs + CL;            // [CL] intra-chunk part of n . q
+  const int b = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int r16 = lane & 15, quad = lane >> 4, col0 = blockIdx.z * 64;
+  const int slot = state_slots[b];
+  const int t_lo = cu_q[b], t_hi = cu_q[b + 1];
+  if (slot < 0) {
+    for (int i = tid; i < (t_hi - t_lo) * 64; i += 256) {
+      const int t = t_lo + i / 64, c = col0 + i % 64;
+      if (c < V) hbuf[((size_t)t * NH + hd) * V + c] = 0.f;
+      if (blockIdx.z == 0 && i % 64 == 0) nq[(size_t)t * NH + hd] = mt[(size_t)t * NH + hd] = 0.f;
+    }
+    return;
+  }
+  if (t_hi <= t_lo) return;
+  const bool fresh = first_pos[b] == 0;
+  const size_t sbase = ((size_t)slot * NH + hd) * D;
+  for (int i = tid; i < DP * 64; i += 256) {
+    const int d = i / 64, c = i % 64;
+    Sst[d * CS + c] = (!fresh && d < D && col0 + c < V) ? S[(sbase + d) * V + col0 + c] : 0.f;
+  }
+  for (int d = tid; d < DP; d += 256) nst[d] = (!fresh && d < D) ? N[sbase + d] : 0.f;
+  float m_prev = fresh ? 0.f : M[(size_t)slot * NH + hd];
+  const float qscale = 1.f / sqrtf((float)D);
+
+  for (int tb = t_lo; tb < t_hi; tb += CL) {
+    const int nt = min(CL, t_hi - tb);
+    __syncthreads();  // the chunk before is done with the staged operands
+    for (int i = tid; i < CL * DP; i += 256) {
+      const int d = i % DP, tt = i / DP;
+      const bool live = tt < nt && d < D;
+      const T* row = proj + (size_t)(tb + min(tt, nt - 1)) * row_stride;
+      Ks[tt * QS + d] = live ? ldf<T>(row, k_off + hd * D + d) : 0.f;
+      Qs[tt * QS + d] = live ? ldf<T>(row, q_off + hd * D + d) * qscale : 0.f;
+    }
+    for (int i = tid; i < CL * 64; i += 256) {
+      const int c = i % 64, tt = i / 64;
+      Vs[tt * CS + c] = (tt < nt && col0 + c < V)
+                            ? ldf<T>(proj + (size_t)(tb + tt) * row_stride, v_off + hd * V + col0 + c) : 0.f;
+    }
+    if (w == 0) {  // running sum of f, running maximum of b = i - F, over the chunk's tokens (lane = token)
+      float F = lane < nt ? fg[(size_t)(tb + lane) * NH + hd] : 0.f;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const float up = __shfl_up(F, o, 64);
+        if (lane >= o) F += up;
+      }
+      const float bb = lane < nt ? ig[(size_t)(tb + lane) * NH + hd] - F : -INFINITY;
+      float g = fmaxf(bb, m_prev);
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const float up = __shfl_up(g, o, 64);
+        if (lane >= o) g = fmaxf(g, up);
+      }
+      Fs[lane] = F;
+      bs[lane] = bb;
+      gs[lane] = g;
+    }
+    __syncthreads();
+    // ---- P[t][s] = exp(b_s - g_t) (q_t . k_s) for s <= t; rows of wave w: t = 16 w + ..
+    {
+      f32x4 c[4];
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb) c[cb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int kk = 0; kk < DP / 4; ++kk) {
+        const float a = Qs[(16 * w + r16) * QS + 4 * kk + quad];
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb)
+          if (cb <= w) c[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Ks[(16 * cb + r16) * QS + 4 * kk + quad], c[cb], 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = 16 * w + 4 * quad + i;
+        const float gt = gs[t];
+        float rs = 0.f;
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) {
+          const int sidx = 16 * cb + r16;
+          const float p = (cb <= w && sidx <= t) ? c[cb][i] * expf(bs[sidx] - gt) : 0.f;
+          Ps[t * CS + sidx] = p;
+          rs += p;
+        }
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) rs += __shfl_xor(rs, o, 64);
+        if (r16 == 0) nqs[t] = rs;
+      }
+    }
+    __syncthreads();
+    // ---- read-out of wave w's tokens: e_t (q_t S_prev) + P V; n . q
+    {
+      f32x4 acc[4];
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb) acc[cb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      const float e_row = expf(m_prev - gs[16 * w + r16]);  // the A operand's row is token 16 w + r16
+      float qn = 0.f;
+      for (int kk = 0; kk < DP / 4; ++kk) {
+        const float qv = Qs[(16 * w + r16) * QS + 4 * kk + quad];
+        qn += qv * nst[4 * kk + quad];
+        const float a = qv * e_row;
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb)
+          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Sst[(4 * kk + quad) * CS + 16 * cb + r16], acc[cb], 0, 0, 0);
+      }
+      for (int kk = 0; kk < 4 * (w + 1); ++kk) {
+        const float a = Ps[(16 * w + r16) * CS + 4 * kk + quad];
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb)
+          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, Vs[(4 * kk + quad) * CS + 16 * cb + r16], acc[cb], 0, 0, 0);
+      }
+      qn += __shfl_xor(qn, 16, 64);  // the four quads hold the key rows 4 kk + quad
+      qn += __shfl_xor(qn, 32, 64);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = 16 * w + 4 * quad + i;
+        if (t < nt) {
+          const size_t th = (size_t)(tb + t) * NH + hd;
+#pragma unroll
+          for (int cb = 0; cb < 4; ++cb) {
+            const int c = col0 + 16 * cb + r16;
+            if (c < V) hbuf[th * V + c] = acc[cb][i];
+          }
+        }
+      }
+      const int tq = 16 * w + r16;  // lanes of quad 0 finish n . q of token 16 w + r16
+      if (blockIdx.z == 0 && quad == 0 && tq < nt) {
+        const size_t th = (size_t)(tb + tq) * NH + hd;
+        nq[th] = e_row * qn + nqs[tq];
+        mt[th] = Fs[tq] + gs[tq];
+      }
+    }
+    __syncthreads();  // every read of the old state is done
+    // ---- state to the end of the chunk
+    {
+      const float gL = gs[CL - 1], decay = expf(m_prev - gL);
+      for (int rb = w; rb < DP / 16; rb += 4) {
+        f32x4 acc[4];
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) acc[cb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int kk = 0; kk < CL / 4; ++kk) {
+          const int sidx = 4 * kk + quad;
+          const float a = Ks[sidx * QS + 16 * rb + r16];
+          const float ws = expf(bs[sidx] - gL);
+#pragma unroll
+          for (int cb = 0; cb < 4; ++cb)
+            acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, ws * Vs[sidx * CS + 16 * cb + r16], acc[cb], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int cb = 0; cb < 4; ++cb) {
+            float* p = Sst + (16 * rb + 4 * quad + i) * CS + 16 * cb + r16;
+            *p = decay * *p + acc[cb][i];
+          }
+      }
+      if (tid < DP) {
+        float a = decay * nst[tid];
+        for (int sidx = 0; sidx < CL; ++sidx) a += expf(bs[sidx] - gL) * Ks[sidx * QS + tid];
+        nst[tid] = a;
+      }
+      m_prev = Fs[CL - 1] + gL;
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < DP * 64; i += 256) {
+    const int d = i / 64, c = i % 64;
+    if (d < D && col0 + c < V) S[(sbase + d) * V + col0 + c] = Sst[d * CS + c];
+  }
+  if (blockIdx.z == 0) {
+    for (int d = tid; d < D; d += 256) N[sbase + d] = nst[d];
+    if (tid == 0) M[(size_t)slot * NH + hd] = m_prev;
+  }
+}
+
 // y = h / (max(|nq|, exp(-m)) + 1e-6); per head: y / rms(y) * w * sigmoid(gate)
 template <typename T>
 __global__ void __launch_bounds__(256) mlstm_out_kernel(const float* __restrict__ hbuf, const float* __restrict__ nq,
@@ -249,10 +449,36 @@ extern "C" int areal_mlstm_gates(const void* x, const void* w, const void* bias,
 extern "C" int areal_mlstm_scan(const void* proj, int64_t row_stride, int q_off, int k_off, int v_off,
                                 const float* ig, const float* fg, const int* cu_q, const int* first_pos,
                                 const int* state_slots, float* S, float* N, float* M, float* hbuf, float* nq,
-                                float* mt, int B, int NH, int D, int V, int dt, hipStream_t st) {
+                                float* mt, int B, int NH, int D, int V, int max_q, int dt, hipStream_t st) {
   if (B == 0) return 0;
   if (D > 256 || D <= 0 || V <= 0) return -1;
   const dim3 grid(B, NH, (V + 63) / 64);
+  if (max_q >= 16 && D <= 128) {  // prompt portions: the chunk-parallel kernel
+#define CHUNK(TT, DPV)                                                                                             \
+  do {                                                                                                             \
+    const size_t lds = sizeof(float) * ((size_t)DPV * (CL + 4) + 2 * (size_t)CL * (DPV + 4) + 2 * (size_t)CL * (CL + 4) + \
+                                        DPV + 4 * CL);                                                             \
+    static bool raised = false;                                                                                    \
+    if (!raised && lds > 64 * 1024) {                                                                              \
+      HIP_RET(hipFuncSetAttribute((const void*)mlstm_chunk_kernel<TT, DPV>,                                        \
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));                        \
+      raised = true;                                                                                               \
+    }                                                                                                              \
+    hipLaunchKernelGGL((mlstm_chunk_kernel<TT, DPV>), grid, dim3(256), lds, st, (const TT*)proj, row_stride, q_off, \
+                       k_off, v_off, ig, fg, cu_q, first_pos, state_slots, S, N, M, hbuf, nq, mt, NH, D, V);       \
+  } while (0)
+#define PICKC(TT)                      \
+  do {                                 \
+    if (D <= 32) CHUNK(TT, 32);        \
+    else if (D <= 64) CHUNK(TT, 64);   \
+    else CHUNK(TT, 128);               \
+  } while (0)
+    if (dt == 0) PICKC(bf16_t);
+    else PICKC(float);
+#undef PICKC
+#undef CHUNK
+    return (int)hipGetLastError();
+  }
 #define LAUNCH(TT, DPV)                                                                                          \
   hipLaunchKernelGGL((mlstm_scan_kernel<TT, DPV>), grid, dim3(64 * RW), 0, st, (const TT*)proj, row_stride, q_off,    \
                      k_off, v_off, ig, fg, cu_q, first_pos, state_slots, S, N, M, hbuf, nq, mt, NH, D, V)

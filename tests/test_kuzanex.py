@@ -134,10 +134,10 @@ def test_window_attention_edges_pages_portions_and_splits(device, dtype, H, G, D
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("NH,D,V", [(3, 24, 40), (1, 8, 8), (2, 64, 72), (2, 130, 16)])
+@pytest.mark.parametrize("NH,D,V", [(3, 24, 40), (1, 8, 8), (2, 64, 72), (2, 130, 16), (2, 128, 128), (2, 48, 64)])
 def test_mlstm_state_carried_over_portions_and_reused_slots(device, dtype, NH, D, V):
     g = torch.Generator().manual_seed(5)
-    n, W, cap, eps = 70, 32, 6.0, 1e-5
+    n, W, cap, eps = 150, 32, 6.0, 1e-5
     x = torch.randn(n, W, generator=g).to(dtype)
     wg = (torch.randn(2 * NH, W, generator=g) * 0.6).to(dtype)
     bg = torch.randn(2 * NH, generator=g).to(dtype)
@@ -164,7 +164,8 @@ def test_mlstm_state_carried_over_portions_and_reused_slots(device, dtype, NH, D
             cu = torch.tensor([0, c], dtype=torch.int32, device=device)
             hb, nq, mt = mlstm_ops.mlstm_scan(pd[at:at + c], 0, NH * D, 2 * NH * D, i_, f_, cu,
                                               torch.tensor([at], dtype=torch.int32, device=device),
-                                              torch.tensor([slot], dtype=torch.int32, device=device), state)
+                                              torch.tensor([slot], dtype=torch.int32, device=device), state,
+                                              max_q=c)  # long portions take the chunk-parallel kernel on the GPU
             outs.append(mlstm_ops.mlstm_out(hb, nq, mt, pd[at:at + c, 2 * NH * D + NH * V:2 * NH * D + 2 * NH * V], nwd,
                                             eps))
             at += c
@@ -174,8 +175,8 @@ def test_mlstm_state_carried_over_portions_and_reused_slots(device, dtype, NH, D
     state.S.fill_(123.0)  # a slot is handed on as it is: a sequence that starts at position 0 must not see this
     state.n.fill_(-7.0)
     state.m.fill_(3.0)
-    assert rel_err(run([2, 9, 1, 1, 17, 8, 30, 2], 1), want) < tol(dtype)
-    assert rel_err(run([40] + [1] * 30, 2), want) < tol(dtype)
+    assert rel_err(run([2, 9, 1, 1, 17, 8, 30, 2, 64, 16], 1), want) < tol(dtype)
+    assert rel_err(run([40, 65] + [1] * 45, 2), want) < tol(dtype)
     # a row without a slot is skipped and leaves every slot alone
     before = state.S.clone()
     i_, f_ = mlstm_ops.mlstm_gates(xd[:4].contiguous(), wgd, bgd, NH, cap)
