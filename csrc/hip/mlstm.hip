@@ -227,6 +227,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(
   float* bs = Fs + CL;             // [CL]
   float* gs = bs + CL;             // [CL]
   float* nqs = gs + CL;            // [CL] intra-chunk part of n . q
+  float* wsl = nqs + CL;           // [CL] exp(b_s - g_L): weight of token s in the state at the chunk's end
   const int b = blockIdx.x, hd = blockIdx.y, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, quad = lane >> 4, col0 = blockIdx.z * 64;
   const int slot = state_slots[b];
@@ -253,12 +254,25 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(
   for (int tb = t_lo; tb < t_hi; tb += CL) {
     const int nt = min(CL, t_hi - tb);
     __syncthreads();  // the chunk before is done with the staged operands
-    for (int i = tid; i < CL * DP; i += 256) {
-      const int d = i % DP, tt = i / DP;
-      const bool live = tt < nt && d < D;
-      const T* row = proj + (size_t)(tb + min(tt, nt - 1)) * row_stride;
-      Ks[tt * QS + d] = live ? ldf<T>(row, k_off + hd * D + d) : 0.f;
-      Qs[tt * QS + d] = live ? ldf<T>(row, q_off + hd * D + d) * qscale : 0.f;
+    if (sizeof(T) == 2 && D == DP && row_stride % 8 == 0 && k_off % 8 == 0 && q_off % 8 == 0) {  // 16-byte loads
+      for (int i = tid; i < CL * DP / 8; i += 256) {
+        const int d = (8 * i) % DP, tt = (8 * i) / DP;
+        const bf16_t* row = reinterpret_cast<const bf16_t*>(proj) + (size_t)(tb + min(tt, nt - 1)) * row_stride;
+        const bf16x8 kx = ld8(row + k_off + hd * D + d), qx = ld8(row + q_off + hd * D + d);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          Ks[tt * QS + d + e] = tt < nt ? bf2f(kx[e]) : 0.f;
+          Qs[tt * QS + d + e] = tt < nt ? bf2f(qx[e]) * qscale : 0.f;
+        }
+      }
+    } else {
+      for (int i = tid; i < CL * DP; i += 256) {
+        const int d = i % DP, tt = i / DP;
+        const bool live = tt < nt && d < D;
+        const T* row = proj + (size_t)(tb + min(tt, nt - 1)) * row_stride;
+        Ks[tt * QS + d] = live ? ldf<T>(row, k_off + hd * D + d) : 0.f;
+        Qs[tt * QS + d] = live ? ldf<T>(row, q_off + hd * D + d) * qscale : 0.f;
+      }
     }
     for (int i = tid; i < CL * 64; i += 256) {
       const int c = i % 64, tt = i / 64;
@@ -282,6 +296,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(
       Fs[lane] = F;
       bs[lane] = bb;
       gs[lane] = g;
+      wsl[lane] = expf(bb - __shfl(g, 63, 64));
     }
     __syncthreads();
     // ---- P[t][s] = exp(b_s - g_t) (q_t . k_s) for s <= t; rows of wave w: t = 16 w + ..
@@ -289,6 +304,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(
       f32x4 c[4];
 #pragma unroll
       for (int cb = 0; cb < 4; ++cb) c[cb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
       for (int kk = 0; kk < DP / 4; ++kk) {
         const float a = Qs[(16 * w + r16) * QS + 4 * kk + quad];
 #pragma unroll
@@ -320,6 +336,7 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(
       for (int cb = 0; cb < 4; ++cb) acc[cb] = (f32x4){0.f, 0.f, 0.f, 0.f};
       const float e_row = expf(m_prev - gs[16 * w + r16]);  // the A operand's row is token 16 w + r16
       float qn = 0.f;
+#pragma unroll 4
       for (int kk = 0; kk < DP / 4; ++kk) {
         const float qv = Qs[(16 * w + r16) * QS + 4 * kk + quad];
         qn += qv * nst[4 * kk + quad];
@@ -363,10 +380,11 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(
         f32x4 acc[4];
 #pragma unroll
         for (int cb = 0; cb < 4; ++cb) acc[cb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
         for (int kk = 0; kk < CL / 4; ++kk) {
           const int sidx = 4 * kk + quad;
           const float a = Ks[sidx * QS + 16 * rb + r16];
-          const float ws = expf(bs[sidx] - gL);
+          const float ws = wsl[sidx];
 #pragma unroll
           for (int cb = 0; cb < 4; ++cb)
             acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, ws * Vs[sidx * CS + 16 * cb + r16], acc[cb], 0, 0, 0);
@@ -381,7 +399,8 @@ __global__ void __launch_bounds__(256) mlstm_chunk_kernel(
       }
       if (tid < DP) {
         float a = decay * nst[tid];
-        for (int sidx = 0; sidx < CL; ++sidx) a += expf(bs[sidx] - gL) * Ks[sidx * QS + tid];
+#pragma unroll 8
+        for (int sidx = 0; sidx < CL; ++sidx) a += wsl[sidx] * Ks[sidx * QS + tid];
         nst[tid] = a;
       }
       m_prev = Fs[CL - 1] + gL;
@@ -457,7 +476,7 @@ extern "C" int areal_mlstm_scan(const void* proj, int64_t row_stride, int q_off,
 #define CHUNK(TT, DPV)                                                                                             \
   do {                                                                                                             \
     const size_t lds = sizeof(float) * ((size_t)DPV * (CL + 4) + 2 * (size_t)CL * (DPV + 4) + 2 * (size_t)CL * (CL + 4) + \
-                                        DPV + 4 * CL);                                                             \
+                                        DPV + 5 * CL);                                                             \
     static bool raised = false;                                                                                    \
     if (!raised && lds > 64 * 1024) {                                                                              \
       HIP_RET(hipFuncSetAttribute((const void*)mlstm_chunk_kernel<TT, DPV>,                                        \
