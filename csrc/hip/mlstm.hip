@@ -58,11 +58,11 @@ __global__ void __launch_bounds__(256) mlstm_gates_kernel(const T* __restrict__ 
   }
 }
 
-constexpr int TC = 8;  // tokens staged per round
+constexpr int TC = 8;  // tokens staged per step of the loop
 constexpr int RW = 4;  // waves of a workgroup: each keeps a quarter of the state's rows
 
 // One workgroup per (row, head, 64 value columns). Wave r keeps rows r DQ .. r DQ + DQ - 1 of S (lane c: column c) and
-// of n (lane i: row i of its quarter) in registers. Per round of TC tokens every wave forms its partial read-outs,
+// of n (lane i: row i of its quarter) in registers. Per step of TC tokens every wave forms its partial read-outs,
 // the partials meet in LDS and wave r finishes tokens r and r + RW.
 template <typename T, int DP>
 __global__ void __launch_bounds__(64 * RW) mlstm_scan_kernel(
@@ -99,8 +99,8 @@ __global__ void __launch_bounds__(64 * RW) mlstm_scan_kernel(
   float nn = (!fresh && nlive) ? N[sbase + nd] : 0.f;
   float m = fresh ? 0.f : M[(size_t)slot * NH + hd];
   const float qscale = 1.f / sqrtf((float)D);
-  // operands of a round are fetched into registers one round ahead, so the loads' latency runs under the
-  // recurrence of the round before
+  // operands of TC tokens are fetched into registers one step ahead, so the loads' latency runs under the
+  // recurrence of the tokens before
   constexpr int KQN = (TC * DP + 64 * RW - 1) / (64 * RW);
   float pk[KQN], pq[KQN], pv[TC], pf[TC], pi[TC];
   auto fetch = [&](int tb) {
@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(64 * RW) mlstm_scan_kernel(
   fetch(t_lo);
   for (int tb = t_lo; tb < t_hi; tb += TC) {
     const int nt = min(TC, t_hi - tb);
-    __syncthreads();  // the round before is finished with kq and the partials
+    __syncthreads();  // the step before is finished with kq and the partials
 #pragma unroll
     for (int j = 0; j < KQN; ++j) {
       const int i = tid + j * 64 * RW;

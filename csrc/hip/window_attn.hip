@@ -135,7 +135,7 @@ __global__ void __launch_bounds__(256) window_attn_kernel(
     const int jb = pg * PAGE;
     // ---- shaped scores of every head
     for (int c = 0; c < G; ++c) {
-      __syncthreads();  // Kt free (and, first time round, the tile set-up visible)
+      __syncthreads();  // Kt free (and, at the first page, the tile set-up visible)
       const T* kp = kcache + ((page * G + c) * PAGE) * D;
       if (sizeof(T) == 2 && D % 8 == 0) {  // 16-byte loads
         for (int i = tid; i < PAGE * D / 8; i += 256) {

@@ -420,7 +420,7 @@ def test_served_from_a_checkpoint_directory(device, tmp_path):
         eng.destroy()
 
 
-def test_config_reader_and_checkpoint_round_trip(tmp_path):
+def test_config_reader_and_checkpoint_save_then_load(tmp_path):
     cfg = ModelConfig.from_hf_dict(SHAPES[1])
     assert cfg.family == "kuzanex" and cfg.n_layers == 3 and cfg.has_recurrent_state
     from areal_vllm_amd.models import build_model
