@@ -71,7 +71,8 @@ def _attention_reference(qn, kn, v, scale, softcap, talk, window):
 @pytest.mark.parametrize("H,G,D,V,window", [(4, 2, 16, 24, 37), (3, 3, 8, 8, 32), (6, 1, 40, 16, 5), (2, 2, 64, 64, 0),
                                             # head sizes the matrix-core kernel takes (bf16 rows of several queries)
                                             (4, 2, 64, 64, 37), (16, 4, 128, 128, 70), (8, 8, 128, 64, 33),
-                                            (2, 1, 64, 128, 0), (6, 2, 64, 64, 40), (12, 4, 64, 64, 45)])
+                                            (2, 1, 64, 128, 0), (6, 2, 64, 64, 40), (12, 4, 64, 64, 45), (5, 1, 64, 64, 20),
+                                            (1, 1, 64, 64, 9)])
 def test_window_attention_edges_pages_portions_and_splits(device, dtype, H, G, D, V, window):
     """A key that dominates its query's scores sits just inside and just outside the window, on both sides of page
     borders and at position 0; whole prompt, portions down to two tokens and split decoding must all agree."""
