@@ -227,6 +227,9 @@ class NativeTrainEngine(TrainEngine):
                 chunks = [stage_layer_range(mc.n_layers, g.pp * g.vpp, c * g.pp + g.coord.pp) for c in range(g.vpp)]
             else:
                 lr = stage_layer_range(mc.n_layers, g.pp, g.coord.pp)
+        if getattr(mc, "layers", None) is not None:
+            raise NotImplementedError(f"the {mc.family} family is served by the rollout engine only: its mechanisms "
+                                      "have no backward pass in the trainer")
         self.model = Transformer(
             mc, dtype=dtype, device=self.device, tp_size=g.tp, tp_rank=g.coord.tp, tp_group=g.group("tp"),
             layer_range=lr, layer_chunks=chunks, has_embed=g.coord.pp == 0, has_head=g.coord.pp == g.pp - 1,

@@ -40,6 +40,39 @@ __global__ void __launch_bounds__(256) scaled_add_norm_kernel(const float* x, co
   }
 }
 
+// Rows of up to 256 * NV elements: the sums stay in registers between the two passes (one read and one write of
+// the stream instead of two of each).
+template <typename T, int NV>
+__global__ void __launch_bounds__(256) scaled_add_norm_reg_kernel(const float* x, const T* __restrict__ y,
+                                                                   const T* __restrict__ gain, float* out32,
+                                                                   T* __restrict__ outc, int W, float alpha,
+                                                                   float eps) {
+  __shared__ float red[16];
+  const size_t row = (size_t)blockIdx.x * W;
+  float z[NV], ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    z[j] = 0.f;
+    if (i < W) {
+      z[j] = alpha * x[row + i];
+      if (y) z[j] += ldf<T>(y, row + i);
+      ss += z[j] * z[j];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float r = ldf<T>(gain, 0) / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    if (i < W) {
+      const float v = z[j] * r;
+      out32[row + i] = v;
+      if (outc) stf<T>(outc, row + i, v);
+    }
+  }
+}
+
 DEVINL float softplusf(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
 template <typename T>
@@ -60,12 +93,20 @@ extern "C" int areal_scaled_add_norm(const float* x, const void* y, const void* 
                                      int T, int W, float alpha, float eps, int dt, hipStream_t st) {
   if (T == 0) return 0;
   if (W <= 0) return -1;
-  if (dt == 0)
-    hipLaunchKernelGGL(scaled_add_norm_kernel<bf16_t>, dim3(T), dim3(256), 0, st, x, (const bf16_t*)y,
-                       (const bf16_t*)gain, out32, (bf16_t*)outc, W, alpha, eps);
-  else
-    hipLaunchKernelGGL(scaled_add_norm_kernel<float>, dim3(T), dim3(256), 0, st, x, (const float*)y,
-                       (const float*)gain, out32, (float*)outc, W, alpha, eps);
+#define LAUNCH(KERNEL, TT)                                                                                       \
+  hipLaunchKernelGGL(KERNEL, dim3(T), dim3(256), 0, st, x, (const TT*)y, (const TT*)gain, out32, (TT*)outc, W, alpha, eps)
+#define PICK(TT)                                                                  \
+  do {                                                                            \
+    if (W <= 256 * 4) LAUNCH((scaled_add_norm_reg_kernel<TT, 4>), TT);            \
+    else if (W <= 256 * 8) LAUNCH((scaled_add_norm_reg_kernel<TT, 8>), TT);       \
+    else if (W <= 256 * 16) LAUNCH((scaled_add_norm_reg_kernel<TT, 16>), TT);     \
+    else if (W <= 256 * 32) LAUNCH((scaled_add_norm_reg_kernel<TT, 32>), TT);     \
+    else LAUNCH(scaled_add_norm_kernel<TT>, TT);                                  \
+  } while (0)
+  if (dt == 0) PICK(bf16_t);
+  else PICK(float);
+#undef PICK
+#undef LAUNCH
   return (int)hipGetLastError();
 }
 

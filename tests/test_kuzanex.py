@@ -43,7 +43,7 @@ def rel_err(got, want):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_scaled_add_norm_and_xielu(device, dtype):
     g = torch.Generator().manual_seed(3)
-    for T, W in ((5, 48), (3, 257), (1, 8)):
+    for T, W in ((5, 48), (3, 257), (1, 8), (2, 1030), (1, 2100), (1, 4100), (1, 8200)):  # every kernel variant
         x = torch.randn(T, W, generator=g)
         y = torch.randn(T, W, generator=g).to(dtype)
         gain = torch.tensor([1.37]).to(dtype)
