@@ -360,6 +360,51 @@ def test_other_sizes_windows_and_layer_orders(device, dtype, which):
         eng.destroy()
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_shapes_orders_and_schedules(device, seed):
+    """Random layer lists (sizes, head layouts, windows, constants, with and without feed-forward) fed through random
+    schedules of up to three live requests: portions of 1 .. 100 tokens, requests that skip steps; 32-bit, so that
+    any deviation beyond rounding shows."""
+    import random
+
+    rng = random.Random(seed)
+    for case in range(3):
+        width, vocab, layers = rng.choice([32, 48, 72]), rng.choice([37, 101]), []
+        for _ in range(rng.randint(1, 4)):
+            ff = rng.choice([0, 40, width])
+            if rng.random() < 0.5:
+                G = rng.choice([1, 2, 3])
+                H = G * rng.choice([1, 2, 4])
+                D = rng.choice([8, 24, 64])
+                V = rng.choice([64, 128]) if D == 64 else rng.choice([8, 40])
+                layers.append(attn_layer(H, G, D, V, rng.choice([1, 2, 31, 32, 33, 100, 0]), ff,
+                                         scale=rng.choice([0.1, 0.3]), softcap=rng.choice([3.0, 50.0])))
+            else:
+                layers.append(mlstm_layer(rng.choice([1, 2, 3]), rng.choice([8, 24, 64, 136]), rng.choice([8, 40, 72]),
+                                          rng.choice([4.0, 12.0]), ff))
+        cfg = config(layers, width=width, vocab=vocab, alpha=rng.choice([0.8, 2.5]), eps=rng.choice([1e-5, 1e-6]))
+        reqs = {f"q{i}": tokens_of(rng.choice([1, 2, 17, 97, 150]), vocab, 100 * case + i)
+                for i in range(rng.randint(1, 3))}
+        at, steps = {r: 0 for r in reqs}, []
+        while any(at[r] < len(t) for r, t in reqs.items()):
+            step = []
+            for r, t in reqs.items():
+                if at[r] < len(t) and rng.random() > 0.2:
+                    c = min(rng.choice([1, 1, 1, 2, 3, 16, 31, 33, 64, 100]), len(t) - at[r])
+                    step.append((r, t[at[r]:at[r] + c], list(range(c)), at[r] + c == len(t)))
+                    at[r] += c
+            if step:
+                steps.append(step)
+        eng, w = make_engine(cfg, device, "float32", num_pages=24, max_running=3)
+        try:
+            got = replay(eng, steps)
+            for r, t in reqs.items():
+                check_against_oracle(got, t, w, cfg, "float32", r)
+        finally:
+            eng.destroy()
+
+
 @pytest.mark.parametrize("device,dtype", CASES)
 def test_first_tokens_and_long_decoding(device, dtype):
     cfg = config([attn_layer(4, 2, 16, 24, 40), mlstm_layer()])
