@@ -155,8 +155,15 @@ class NativeInferenceEngine:
         if hybrid:
             assert not kv_fp8, "layer-list decoders keep their caches in the model's dtype"
             elt = torch.empty((), dtype=self.dtype).element_size()
-            per_page = max(1, sum(g * (d + v) for g, d, v in (blk.mix.cache_shape() for blk in self.model.layers
-                                                             if blk.kind == "attention")) * PAGE_SIZE * elt)
+            per_tok = 0  # cached numbers per token, over all layer runs
+            for li in getattr(self.model, "layer_runs", range(len(self.model.layers))):
+                blk = self.model.layers[li]
+                if blk.kind == "attention":
+                    g, d, v = blk.mix.cache_shape()
+                    per_tok += g * (d + v)
+                elif blk.kind == "latent_attention":
+                    per_tok += sum(blk.mix.cache_shape())
+            per_page = max(1, per_tok * PAGE_SIZE * elt)
         else:
             hkv = self.model.layers[0].attn.hkv
             per_page = _kv_bytes_per_page(mc, len(self.model.layers), hkv, 1 if kv_fp8 else 2)

@@ -100,6 +100,12 @@ class ModelRunner:
         self.fused_qkv_rope = (cfg.head_dim % 64 == 0 and not cfg.qk_norm
                                and os.environ.get("AREAL_FUSED_QKV_ROPE", "1") != "0")
 
+    keeps_positions = False  # runners whose layers rotate by position themselves keep the plan's positions
+
+    def _embed(self, ids: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
+        """Token ids of a plan -> what the layer loop starts from."""
+        return self.model.embed_tokens(ids, pos)
+
     def _alloc_caches(self, kv_dtype):
         cfg, model = self.cfg, self.model
         self.hq = model.layers[0].attn.hq
@@ -312,9 +318,9 @@ class ModelRunner:
             rope = self.model.mrope(pos3)  # per-token table, addressed by the token's index in the plan
             pos = torch.arange(T, dtype=torch.int32, device=dev)
         else:
-            h = self.model.embed_tokens(ids, pos)
+            h = self._embed(ids, pos)
         if self.cfg.pos_embed != "rope":
-            pos = torch.zeros_like(pos)  # the only row of the angle-zero table
+            pos = torch.zeros_like(pos) if not self.keeps_positions else pos  # the only row of the angle-zero table
         h, residual = self._prefill_layers(plan, h, pos, slots, rope, cu_q, cu_k, bt, max_q)
         if plan.get("logit_rows") is not None:  # scoring: fp32 logits at chosen tokens of the packed batch
             rows = torch.from_numpy(np.asarray(plan["logit_rows"], dtype=np.int64)).to(dev)
@@ -598,7 +604,7 @@ class ModelRunner:
         ops.decode_begin_(st["kill"], st["active"], st["positions"], st["context_lens"], st["slots"],
                           st["block_tables"])
         for s in range(self.decode_steps):
-            h = self.model.embed_tokens(st["input_ids"], st["positions"])
+            h = self._embed(st["input_ids"], st["positions"])
             rope_pos = st["positions"] if self.cfg.pos_embed == "rope" else st["zero_pos"]
             if self.is_vl:  # generated tokens of a request with images sit `delta` away from their index
                 torch.add(st["positions"], st["rope_delta"], out=st["rope_pos"])
@@ -855,26 +861,54 @@ class HybridModelRunner(ModelRunner):
         self.plain_family = True
 
     def _alloc_caches(self, kv_dtype):
+        from ..ops import latent_attention as lattn
         from ..ops import mlstm as mlstm_ops
         from ..ops import window_attention as wattn
 
         assert kv_dtype is None, "layer-list decoders keep their caches in the model's dtype"
         self.hq = self.hkv = 1
+        self.sandwich = bool(getattr(self.model, "sandwich", False))
+        self.keeps_positions = self.sandwich
+        # one cache / state per layer RUN: a layer that runs several times keeps every pass apart
+        self.layer_runs = list(getattr(self.model, "layer_runs", range(len(self.model.layers))))
         self.kv, self.state = [], []
-        for blk in self.model.layers:
+        tables: Dict[Any, torch.Tensor] = {}
+        for li in self.layer_runs:
+            blk = self.model.layers[li]
             if blk.kind == "attention":
                 G, D, V = blk.mix.cache_shape()
                 self.kv.append(wattn.alloc_window_cache(self.num_pages, G, D, V, self.dtype, self.device))
                 self.state.append(None)
+            elif blk.kind == "latent_attention":
+                R, P = blk.mix.cache_shape()
+                blk.mix.prepare(self.max_context + 1, tables)
+                self.kv.append(lattn.alloc_latent_cache(self.num_pages, R, P, self.dtype, self.device))
+                hist = blk.state_shape()  # the input convolution's last inputs, per request slot
+                self.state.append(torch.zeros(self.n_state_slots, *hist, dtype=torch.float32, device=self.device)
+                                  if hist else None)
             else:
                 H, D, V = blk.mix.state_shape()
                 self.kv.append(None)
                 self.state.append(mlstm_ops.RecurrentState(self.n_state_slots, H, D, V, self.device))
+        # designs whose embedding looks at the token before: the last token of every request slot
+        self.prev_tokens = (torch.zeros(self.n_state_slots, dtype=torch.int32, device=self.device)
+                            if getattr(self.model, "bigram", None) is not None else None)
         self._neg1 = torch.full((1,), -1, dtype=torch.int32, device=self.device)
 
+    def _embed(self, ids: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
+        if self.sandwich:  # the embedding needs the rows of the plan: `_run_layers` computes it
+            return ids
+        return self.model.embed_tokens(ids, pos)
+
     def kv_cache_bytes(self) -> int:
-        return (sum(k.numel() * k.element_size() + v.numel() * v.element_size() for k, v in filter(None, self.kv))
-                + sum(s.nbytes() for s in self.state if s is not None))
+        n = 0
+        for c in self.kv:
+            for t in (c if isinstance(c, tuple) else (c,)):
+                n += t.numel() * t.element_size() if t is not None else 0
+        for s in self.state:
+            if s is not None:
+                n += s.nbytes() if hasattr(s, "nbytes") and callable(s.nbytes) else s.numel() * s.element_size()
+        return n
 
     # ------------------------------------------------------------------------------ layers
     def _run_layers(self, xc: torch.Tensor, st) -> torch.Tensor:
@@ -882,11 +916,14 @@ class HybridModelRunner(ModelRunner):
         from ..ops.post_norm import scaled_add_norm
 
         cfg = self.cfg
+        if self.sandwich:
+            return self._run_layers_sandwich(xc, st)
         x32 = xc.float() if xc.dtype != torch.float32 else xc.clone()
         alpha, eps = float(cfg.postln_alpha), float(cfg.rms_norm_eps)
         trace = getattr(self, "layer_trace", None)
-        for li, blk in enumerate(self.model.layers):
-            y = blk.mix.step(xc, st, self.kv[li] if blk.kind == "attention" else self.state[li])
+        for ri, li in enumerate(self.layer_runs):
+            blk = self.model.layers[li]
+            y = blk.mix.step(xc, st, self.kv[ri] if blk.kind == "attention" else self.state[ri])
             x32, xc = scaled_add_norm(x32, y, blk.norm1, alpha, eps, self.dtype)
             if blk.norm2 is not None:
                 y = blk.mlp(xc) if blk.mlp is not None else None
@@ -895,9 +932,40 @@ class HybridModelRunner(ModelRunner):
                 trace.append(x32.clone())
         return x32
 
+    def _run_layers_sandwich(self, ids: torch.Tensor, st) -> torch.Tensor:
+        """Token ids -> fp32 residual stream after the last layer run. Every sublayer's closing kernel (gate, norm,
+        scale, residual sum) also produces the norm that the next sublayer reads; the last one leaves the stream to
+        the final norm."""
+        from ..ops import sandwich as sw
+
+        model, eps = self.model, float(self.cfg.rms_norm_eps)
+        f32 = self.dtype == torch.float32
+        x32 = model.embed_step(ids, st, self.prev_tokens)
+        blocks = [model.layers[li] for li in self.layer_runs]
+        trace = getattr(self, "layer_trace", None)
+        h32 = hc = None
+        for ri, blk in enumerate(blocks):
+            if h32 is None and hc is None:
+                h32, hc = sw.layer_norm(x32, blk.norm1, blk.norm1_bias, eps, self.dtype,
+                                        want32=f32 or blk.canon1 is not None)
+            nxt = blocks[ri + 1] if ri + 1 < len(blocks) else None
+            x32, h32, hc = blk.step(x32, h32, hc, st, self.kv[ri], self.state[ri],
+                                    (nxt.norm1, nxt.norm1_bias) if nxt is not None else None)
+            if trace is not None:
+                trace.append(x32.clone())
+        return x32
+
     def _final_logits(self, h, residual, fp32: bool = False) -> torch.Tensor:
         from ..ops.post_norm import scaled_add_norm
 
+        if self.sandwich:
+            from ..ops import sandwich as sw
+
+            x32, xc = sw.layer_norm(h.contiguous(), self.model.norm, self.model.norm_bias,
+                                    float(self.cfg.rms_norm_eps), self.dtype)
+            if fp32 or self.keep_logits:
+                return F.linear(x32, self.model.head_weight.float())
+            return F.linear(xc, self.model.head_weight)
         x32, xc = scaled_add_norm(h.contiguous(), None, self.model.norm, 1.0, float(self.cfg.rms_norm_eps),
                                   self.dtype, inplace=False)
         if fp32 or self.keep_logits:
@@ -913,10 +981,10 @@ class HybridModelRunner(ModelRunner):
         first = plan["positions"][plan["cu_q"][:-1]].astype(np.int32)
         ss = plan.get("state_slots")
         ss = np.asarray(ss, dtype=np.int32) if ss is not None and len(ss) == B else np.full(B, -1, np.int32)
-        if any(s is not None for s in self.state):
+        if any(s is not None for s in self.state) or self.prev_tokens is not None:
             assert (ss >= 0).all() and (ss < self.n_state_slots).all(), "a row of the plan has no state slot"
         st = StepTensors(cu_q, torch.from_numpy(plan["chunk_end"].astype(np.int32)).to(dev), max_q, slots, bt,
-                         torch.from_numpy(first).to(dev), torch.from_numpy(ss).to(dev))
+                         torch.from_numpy(first).to(dev), torch.from_numpy(ss).to(dev), positions=pos)
         return self._run_layers(h, st), None
 
     # ------------------------------------------------------------------------------ decode
@@ -924,6 +992,15 @@ class HybridModelRunner(ModelRunner):
         from ..ops import window_attention as wattn
 
         nsplit, ws = 1, None
+        latent = [blk.mix for blk in self.model.layers if blk.kind == "latent_attention"]
+        if latent and self.device.type == "cuda":
+            from ..ops import latent_attention as lattn
+
+            nsplit = max(lattn.decode_splits(Bp, m.window, self.max_context) for m in latent)
+            if nsplit > 1:
+                ws = (torch.empty(Bp * nsplit * max(m.H * m.R for m in latent), dtype=torch.float32, device=self.device),
+                      torch.empty(Bp * nsplit * max(m.H for m in latent) * 2, dtype=torch.float32, device=self.device))
+            return nsplit, ws
         mixers = [blk.mix for blk in self.model.layers if blk.kind == "attention"]
         if mixers and self.device.type == "cuda":
             nsplit = max(wattn.decode_splits(Bp, m.shape.window, self.max_context) for m in mixers)
@@ -943,5 +1020,5 @@ class HybridModelRunner(ModelRunner):
         # rows that are retired (no cache slot) touch no state slot either
         eff = torch.where(st["slots"] < 0, self._neg1, st["state_slots"])
         step = StepTensors(st["cu_rows"], st["context_lens"], 1, st["slots"], st["block_tables"], st["positions"], eff,
-                           nsplit=st["nsplit"], workspace=st["ws"])
+                           nsplit=st["nsplit"], workspace=st["ws"], positions=st["positions"])
         return self._final_logits(self._run_layers(h, step), None)

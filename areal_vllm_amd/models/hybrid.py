@@ -6,9 +6,17 @@ Layer:      x <- norm1(alpha x + mixer(x));  x <- norm2(alpha x + ff(x))       (
 Norm:       z / sqrt(mean(z^2) + eps) * g, g one number.
 Output:     logits = head . norm(x).
 
+The Lufivik design is the second member. Its layers sit between two norms each (layer norm with bias):
+
+Layer:      h = norm1(x); x <- x + s1 * norm1b(mixer(h + conv(h)) * sigmoid(W_r1 h + b_r1));  the same around ff
+Mixer:      attention through a shared low-rank latent (the cache holds the latent and one rotated key per token)
+ff:         routed experts, gated units with clamped pre-activations, softmax router weights as they are
+Embedding:  token plus hashed-bigram row, then a norm;  a span of layers may run several times (own caches per pass)
+
 The mechanisms are separate modules with their constants as constructor arguments (``WindowAttentionMixer``,
-``MLSTMMixer``, ``XieluMLP``); what they compute is documented with their kernels (``ops/window_attention.py``,
-``ops/mlstm.py``, ``ops/post_norm.py``). The modules hold parameters and know how to run ONE step on the tensors of a
+``MLSTMMixer``, ``XieluMLP``, ``LatentAttentionMixer``, ``RoutedGLUExperts``); what they compute is documented with
+their kernels (``ops/window_attention.py``, ``ops/mlstm.py``, ``ops/post_norm.py``, ``ops/latent_attention.py``,
+``ops/sandwich.py``). The modules hold parameters and know how to run ONE step on the tensors of a
 batch plan; paged caches, state slots and the loop over layers belong to the model runner
 (``inference/model_runner.py::HybridModelRunner``).
 """
@@ -23,7 +31,10 @@ import torch.nn.functional as F
 
 from .. import ops
 from ..ops import mlstm as mlstm_ops
-from ..ops import post_norm, window_attention as wattn
+from ..ops import latent_attention as lattn
+from ..ops import moe as moe_ops
+from ..ops import post_norm, sandwich, window_attention as wattn
+from ..ops.grouped_gemm import grouped_gemm_rows
 from .config import ModelConfig
 from .transformer import FlatParams
 
@@ -34,12 +45,28 @@ class HybridConfig(ModelConfig):
     "mlp": {"kind": "dense", "ff": F} | None}, as the checkpoint's config.json lists them."""
     layers: List[Dict[str, Any]] = dataclasses.field(default_factory=list)
     postln_alpha: float = 1.0
+    design: str = "Kuzanex"
+    block_style: str = "post_norm"  # "post_norm": norm after every sum; "sandwich": norms before and after a sublayer
+    loop: Optional[Dict[str, int]] = None  # layers start .. stop - 1 run `times` times in a row
+    canon_taps: int = 0  # taps of the causal convolution on a mixer's input (0: none)
+    bigram: Optional[Dict[str, int]] = None  # hashed-bigram embedding: buckets, mul_prev, mul_cur
 
     @property
     def has_recurrent_state(self) -> bool:
-        return any(l["type"] == "mlstm" for l in self.layers)
+        return any(l["type"] == "mlstm" for l in self.layers) or self.canon_taps > 1 or self.bigram is not None
+
+    @property
+    def layer_runs(self) -> List[int]:
+        """Index of the layer whose weights each layer run uses, in execution order."""
+        n = len(self.layers)
+        if not self.loop:
+            return list(range(n))
+        a, b, k = int(self.loop["start"]), int(self.loop["stop"]), int(self.loop["times"])
+        return list(range(a)) + list(range(a, b)) * k + list(range(b, n))
 
     def n_params(self, with_embedding: bool = True) -> int:
+        if self.block_style == "sandwich":
+            return self._n_params_sandwich(with_embedding)
         W, n = self.hidden_size, 1
         for l in self.layers:
             m = l["mixer"]
@@ -54,7 +81,32 @@ class HybridConfig(ModelConfig):
                 n += 2 * W * l["mlp"]["ff"] + W + l["mlp"]["ff"] + 3
         return n + (2 * self.vocab_size * W if with_embedding else 0)
 
+    def _n_params_sandwich(self, with_embedding: bool) -> int:
+        W = self.hidden_size
+        n = 4 * W  # embedding norm, final norm
+        for l in self.layers:
+            m = l["mixer"]
+            H, D, P, V, Q, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["q_rank"], m["kv_rank"]
+            n += W * (Q + R + P + H) + Q + R + Q * H * (D + P) + R * H * (D + V) + W * H * V
+            n += 5 * W + W * W + W + W * max(0, self.canon_taps)
+            if l.get("mlp"):
+                e = l["mlp"]
+                n += e["router"]["experts"] * (W + 3 * W * e["expert"]["ff"]) + 5 * W + W * W + W
+        if with_embedding:
+            n += 2 * self.vocab_size * W + ((self.bigram["buckets"] + 1) * W if self.bigram else 0)
+        return n
+
     def to_hf_dict(self) -> Dict[str, Any]:
+        if self.block_style == "sandwich":
+            d = {"architecture": self.design, "layers": [dict(l) for l in self.layers],
+                 "norm": {"eps": self.rms_norm_eps}, "vocab": self.vocab_size, "width": self.hidden_size}
+            if self.canon_taps:
+                d["canon"] = {"taps": self.canon_taps}
+            if self.bigram:
+                d["embedding"] = {"bigram": dict(self.bigram)}
+            if self.loop:
+                d["loop"] = dict(self.loop)
+            return d
         layers = [{k: v for k, v in l.items() if k != "second_norm" or v} for l in self.layers]
         return {"architecture": "Kuzanex", "layers": layers, "norm": {"eps": self.rms_norm_eps},
                 "postln_alpha": self.postln_alpha, "vocab": self.vocab_size, "width": self.hidden_size}
@@ -99,15 +151,56 @@ def kuzanex_config_from_dir(path: str) -> HybridConfig:
     return cfg
 
 
+def lufivik_config(d: Dict[str, Any]) -> HybridConfig:
+    """config.json of a Lufivik checkpoint -> HybridConfig. Every size and constant is taken from it."""
+    layers = []
+    for i, l in enumerate(d["layers"]):
+        if l["type"] != "latent_attention":
+            raise ValueError(f"layer {i}: unknown mixer type {l['type']!r}")
+        mlp = l.get("mlp")
+        if mlp is not None and mlp.get("kind") != "moe":
+            raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+        m = l["mixer"]
+        if int(m["rot"]["dims"]) != int(m["rot_dim"]) or int(m["rot_dim"]) % 2:
+            raise ValueError(f"layer {i}: the rotary part has rot_dim (an even number of) dimensions")
+        layers.append({"type": l["type"], "mixer": json.loads(json.dumps(m)),
+                       "mlp": json.loads(json.dumps(mlp)) if mlp is not None else None})
+    n = len(layers)
+    loop = d.get("loop")
+    if loop is not None:
+        loop = {k: int(loop[k]) for k in ("start", "stop", "times")}
+        if not (0 <= loop["start"] <= loop["stop"] <= n and loop["times"] >= 1):
+            raise ValueError(f"loop {loop} does not fit {n} layers")
+    big = (d.get("embedding") or {}).get("bigram")
+    m0 = layers[0]["mixer"]
+    moe = [l["mlp"] for l in layers if l["mlp"]]
+    return HybridConfig(
+        family="lufivik", design="Lufivik", block_style="sandwich", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), n_layers=n, n_q_heads=int(m0["heads"]), n_kv_heads=1, head_dim=int(m0["dim"]),
+        intermediate_size=max([e["expert"]["ff"] for e in moe] or [0]), rms_norm_eps=float(d["norm"]["eps"]),
+        max_position_embeddings=int(d.get("max_positions", 1 << 17)), tie_word_embeddings=False, qkv_bias=False,
+        pos_embed="none", norm_type="layer", layers=layers, loop=loop,
+        canon_taps=int((d.get("canon") or {}).get("taps", 0)),
+        bigram={k: int(big[k]) for k in ("buckets", "mul_prev", "mul_cur")} if big else None,
+        eos_token_id=d.get("eos_token_id"), pad_token_id=d.get("pad_token_id"))
+
+
+def lufivik_config_from_dir(path: str) -> HybridConfig:
+    with open(os.path.join(path, "config.json")) as f:
+        return lufivik_config(json.load(f))
+
+
 class StepTensors:
     """What one batch plan hands to the mixers (all on the device): rows of the packed token batch (`cu_q`, longest
     row `max_q`), each row's context length after the step, cache slot of every token, page tables, position of each
     row's first token, state slot of each row, and the decode launch's split count / workspace."""
 
-    def __init__(self, cu_q, ctx_len, max_q, slots, block_tables, first_pos, state_slots, nsplit=1, workspace=None):
+    def __init__(self, cu_q, ctx_len, max_q, slots, block_tables, first_pos, state_slots, nsplit=1, workspace=None,
+                 positions=None):
         self.cu_q, self.ctx_len, self.max_q, self.slots = cu_q, ctx_len, int(max_q), slots
         self.block_tables, self.first_pos, self.state_slots = block_tables, first_pos, state_slots
         self.nsplit, self.workspace = int(nsplit), workspace
+        self.positions = positions  # position of every token (int32), for mixers that rotate by position
 
 
 class WindowAttentionMixer(nn.Module):
@@ -183,6 +276,160 @@ class XieluMLP(nn.Module):
         return F.linear(post_norm.xielu(F.linear(xc, self.up, self.up_bias), self.act), self.down, self.down_bias)
 
 
+class LatentAttentionMixer(nn.Module):
+    """Attention through a shared low-rank latent (``ops/latent_attention.py``): query latent | key/value latent |
+    rotary key part | one gate logit per head come out of ONE projection; the queries are expanded from their
+    normalised latent, their unrotated parts are carried into latent space with the key expansion (so the cache's
+    latents are scored directly) and the attended latents are expanded to values afterwards."""
+
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, q_rank: int, kv_rank: int,
+                 scale: float, window: int, rot_base: float, eps: float, dtype, device):
+        super().__init__()
+        self.H, self.D, self.P, self.V, self.Q, self.R = heads, dim, rot_dim, vdim, q_rank, kv_rank
+        self.scale, self.window, self.rot_base, self.eps = float(scale), int(window), float(rot_base), float(eps)
+        self.proj = nn.Parameter(torch.empty(q_rank + kv_rank + rot_dim + heads, width, dtype=dtype, device=device))
+        self.q_norm = nn.Parameter(torch.ones(q_rank, dtype=dtype, device=device))
+        self.c_norm = nn.Parameter(torch.ones(kv_rank, dtype=dtype, device=device))
+        self.uq = nn.Parameter(torch.empty(heads * (dim + rot_dim), q_rank, dtype=dtype, device=device))
+        self.uk = nn.Parameter(torch.empty(heads * dim, kv_rank, dtype=dtype, device=device))
+        self.uv = nn.Parameter(torch.empty(heads * vdim, kv_rank, dtype=dtype, device=device))
+        self.o = nn.Parameter(torch.empty(width, heads * vdim, dtype=dtype, device=device))
+        self.table: Optional[torch.Tensor] = None  # cosines | sines per position (`prepare`)
+
+    def cache_shape(self):
+        return self.R, self.P
+
+    def prepare(self, n_pos: int, tables: Dict[Any, torch.Tensor]):
+        """The rotation table for positions below `n_pos`; mixers with the same base and size share one."""
+        key = (self.rot_base, self.P, int(n_pos))
+        if key not in tables:
+            tables[key] = lattn.rotary_table(self.rot_base, self.P, int(n_pos), self.proj.device)
+        self.table = tables[key]
+
+    def step(self, hc: torch.Tensor, st: StepTensors, cache: torch.Tensor) -> torch.Tensor:
+        T = hc.shape[0]
+        H, D, P, V, Q, R = self.H, self.D, self.P, self.V, self.Q, self.R
+        proj = F.linear(hc, self.proj)
+        cq = lattn.latent_prep(proj, Q, R, P, self.q_norm, self.c_norm, st.positions, st.slots, cache, self.table,
+                               self.eps)
+        q = F.linear(cq, self.uq).view(T, H, D + P)
+        # q~_h = W_uk[h]^T q^n_h: one batched product over the heads
+        q_lat = torch.bmm(q[:, :, :D].transpose(0, 1), self.uk.view(H, D, R)).transpose(0, 1).contiguous()
+        o_lat = lattn.latent_attention(q, q_lat, cache, st.block_tables, st.cu_q, st.ctx_len, st.max_q, D, P,
+                                       self.scale, self.window, self.table, gate=proj[:, Q + R + P:],
+                                       nsplit=st.nsplit if st.max_q == 1 else 1, workspace=st.workspace)
+        o = torch.bmm(o_lat.transpose(0, 1), self.uv.view(H, V, R).transpose(1, 2)).transpose(0, 1)
+        return F.linear(o.reshape(T, H * V), self.o)
+
+
+class RoutedGLUExperts(nn.Module):
+    """Routed experts without biases: softmax over all router logits (fp32), the `top` largest scores are the
+    weights as they are; expert: down(g sigmoid(alpha g) (u + 1)) with g = min(gate h, limit), u = clamp(up h,
+    -limit, limit). Tokens are sorted by expert and every expert runs on a contiguous slab (grouped kernels, row
+    ranges on the device)."""
+
+    def __init__(self, width: int, ff: int, experts: int, top: int, limit: float, alpha: float, dtype, device):
+        super().__init__()
+        assert 1 <= top <= experts
+        self.E, self.k, self.ff, self.limit, self.alpha = experts, top, ff, float(limit), float(alpha)
+        self.router = nn.Parameter(torch.empty(experts, width, dtype=dtype, device=device))
+        self.gate_up = nn.Parameter(torch.empty(experts, 2 * ff, width, dtype=dtype, device=device))
+        self.down = nn.Parameter(torch.empty(experts, width, ff, dtype=dtype, device=device))
+
+    def forward(self, hc: torch.Tensor, h32: Optional[torch.Tensor]) -> torch.Tensor:
+        if hc.dtype == torch.float32:
+            z = F.linear(hc, self.router)
+        elif hc.is_cuda:  # bf16 operands, fp32 accumulation AND fp32 logits
+            z = torch.mm(hc, self.router.t(), out_dtype=torch.float32)
+        else:
+            z = F.linear(hc.float(), self.router.float())
+        topv, topi = moe_ops.moe_topk(z, self.k, False, out_dtype=torch.float32)
+        order, inv, src_row, offsets = moe_ops.moe_sort(topi.reshape(-1), self.E, self.k)
+        xs = moe_ops._gather_rows(hc, src_row)
+        a = moe_ops.clamped_glu(grouped_gemm_rows(xs, self.gate_up, offsets), self.limit, self.alpha)
+        return moe_ops.combine_rows_w32(grouped_gemm_rows(a, self.down, offsets), inv, topv)
+
+
+class SandwichBlock(nn.Module):
+    """A layer whose sublayers sit between two layer norms, with a sigmoid gate computed from the sublayer's normed
+    input, one scale per channel on the result, and a causal convolution on what the mixer reads."""
+
+    def __init__(self, cfg: HybridConfig, spec: Dict[str, Any], dtype, device):
+        super().__init__()
+        W, m, eps = cfg.hidden_size, spec["mixer"], cfg.rms_norm_eps
+        self.kind, self.eps = spec["type"], float(eps)
+
+        def vec(n=W, one=False):
+            return nn.Parameter((torch.ones if one else torch.zeros)(n, dtype=dtype, device=device))
+
+        mask = m.get("mask") or {}
+        self.mix = LatentAttentionMixer(W, int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]),
+                                        int(m["q_rank"]), int(m["kv_rank"]), float(m["scale"]),
+                                        int(mask.get("size") or 0), float(m["rot"]["base"]), eps, dtype, device)
+        self.norm1, self.norm1_bias, self.norm1b, self.norm1b_bias = vec(one=True), vec(), vec(one=True), vec()
+        self.ls1 = vec(one=True)
+        self.rg1 = nn.Parameter(torch.empty(W, W, dtype=dtype, device=device))
+        self.rg1_bias = vec()
+        self.canon1 = (nn.Parameter(torch.zeros(W, cfg.canon_taps, dtype=dtype, device=device))
+                       if cfg.canon_taps > 0 else None)
+        e = spec.get("mlp")
+        self.mlp = None
+        if e:
+            self.mlp = RoutedGLUExperts(W, int(e["expert"]["ff"]), int(e["router"]["experts"]), int(e["router"]["top"]),
+                                        float(e["expert"]["limit"]), 1.702, dtype, device)
+            self.norm2, self.norm2_bias, self.norm2b, self.norm2b_bias = vec(one=True), vec(), vec(one=True), vec()
+            self.ls2 = vec(one=True)
+            self.rg2 = nn.Parameter(torch.empty(W, W, dtype=dtype, device=device))
+            self.rg2_bias = vec()
+
+    def state_shape(self):
+        """(taps - 1, width) of the convolution's history, or None."""
+        return (self.canon1.shape[1] - 1, self.canon1.shape[0]) if self.canon1 is not None and self.canon1.shape[1] > 1 \
+            else None
+
+    def step(self, x32: torch.Tensor, h32: torch.Tensor, hc: torch.Tensor, st: StepTensors, cache, state,
+             next_norm) -> Any:
+        """x32: the stream; (h32, hc) = norm1(x32) in fp32 and in the compute dtype. Returns the new stream and the
+        `next_norm` (weight, bias) of it, again in both forms."""
+        dtype = hc.dtype
+        gate = F.linear(hc, self.rg1, self.rg1_bias)
+        if self.canon1 is not None:
+            hc = sandwich.canon_conv(h32, self.canon1, state, st.cu_q, st.first_pos, st.state_slots, dtype)
+        y = self.mix.step(hc, st, cache)
+        if self.mlp is None:
+            return sandwich.gated_norm_add(x32, y, gate, self.norm1b, self.norm1b_bias, self.ls1, self.eps, next_norm)
+        x32, h32, hc = sandwich.gated_norm_add(x32, y, gate, self.norm1b, self.norm1b_bias, self.ls1, self.eps,
+                                               (self.norm2, self.norm2_bias), want32=dtype == torch.float32)
+        gate = F.linear(hc, self.rg2, self.rg2_bias)
+        y = self.mlp(hc, h32)
+        return sandwich.gated_norm_add(x32, y, gate, self.norm2b, self.norm2b_bias, self.ls2, self.eps, next_norm)
+
+    def checkpoint_tensors(self, p: str) -> Dict[str, torch.Tensor]:
+        m = self.mix
+        Q, R, P = m.Q, m.R, m.P
+        out = {p + "mix.dq": m.proj.data[:Q], p + "mix.dkv": m.proj.data[Q:Q + R + P],
+               p + "mix.g": m.proj.data[Q + R + P:], p + "mix.dq.norm": m.q_norm.data,
+               p + "mix.dkv.norm": m.c_norm.data, p + "mix.uq": m.uq.data, p + "mix.uk": m.uk.data,
+               p + "mix.uv": m.uv.data, p + "mix.o": m.o.data}
+        for k in ("1", "2") if self.mlp is not None else ("1",):
+            for nm in ("norm" + k, "norm" + k + "b"):
+                out[p + nm] = getattr(self, nm).data
+                out[p + nm + ".b"] = getattr(self, nm + "_bias").data
+            out[p + "ls" + k] = getattr(self, "ls" + k).data
+            out[p + "rg" + k] = getattr(self, "rg" + k).data
+            out[p + "rg" + k + ".b"] = getattr(self, "rg" + k + "_bias").data
+        if self.canon1 is not None:
+            out[p + "canon1"] = self.canon1.data
+        if self.mlp is not None:
+            e, f = self.mlp, self.mlp.ff
+            out[p + "mlp.router"] = e.router.data
+            for i in range(e.E):
+                out[p + f"mlp.e{i}.gate"] = e.gate_up.data[i, :f]
+                out[p + f"mlp.e{i}.up"] = e.gate_up.data[i, f:]
+                out[p + f"mlp.e{i}.down"] = e.down.data[i]
+        return out
+
+
 class HybridBlock(nn.Module):
     def __init__(self, cfg: HybridConfig, spec: Dict[str, Any], dtype, device):
         super().__init__()
@@ -223,8 +470,20 @@ class HybridDecoder(nn.Module):
         self.layer_ids = list(range(cfg.n_layers))
         self.vocab_range = (0, cfg.vocab_size)
         self.embed = nn.Parameter(torch.empty(cfg.vocab_size, cfg.hidden_size, dtype=dtype, device=device))
-        self.layers = nn.ModuleList([HybridBlock(cfg, spec, dtype, device) for spec in cfg.layers])
-        self.norm = nn.Parameter(torch.ones(1, dtype=dtype, device=device))
+        self.sandwich = cfg.block_style == "sandwich"
+        self.layer_runs = cfg.layer_runs
+        if self.sandwich:
+            W = cfg.hidden_size
+            self.bigram = (nn.Parameter(torch.empty(cfg.bigram["buckets"] + 1, W, dtype=dtype, device=device))
+                           if cfg.bigram else None)
+            self.embed_norm = nn.Parameter(torch.ones(W, dtype=dtype, device=device))
+            self.embed_norm_bias = nn.Parameter(torch.zeros(W, dtype=dtype, device=device))
+            self.layers = nn.ModuleList([SandwichBlock(cfg, spec, dtype, device) for spec in cfg.layers])
+            self.norm = nn.Parameter(torch.ones(W, dtype=dtype, device=device))
+            self.norm_bias = nn.Parameter(torch.zeros(W, dtype=dtype, device=device))
+        else:
+            self.layers = nn.ModuleList([HybridBlock(cfg, spec, dtype, device) for spec in cfg.layers])
+            self.norm = nn.Parameter(torch.ones(1, dtype=dtype, device=device))
         self.head = nn.Parameter(torch.empty(cfg.vocab_size, cfg.hidden_size, dtype=dtype, device=device))
         self.flat: Optional[FlatParams] = None
         self.flat_experts = None
@@ -242,7 +501,14 @@ class HybridDecoder(nn.Module):
         W = self.cfg.hidden_size
         for n, p in self.named_parameters():
             leaf = n.rsplit(".", 1)[-1]
-            if leaf == "talk":
+            if self.sandwich and leaf != "embed" and (p.dim() == 1 or leaf == "canon1"):
+                if leaf.endswith("_bias"):
+                    p.data.copy_(0.1 * torch.randn(p.shape, generator=g))
+                elif leaf == "canon1":
+                    p.data.copy_(0.3 * torch.randn(p.shape, generator=g))
+                else:  # norm weights and layer scales
+                    p.data.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=g))
+            elif leaf == "talk":
                 p.data.copy_(torch.eye(p.shape[0]) + 0.1 * torch.randn(p.shape, generator=g))
             elif leaf in ("norm1", "norm2") or n == "norm" or leaf in ("q_norm", "k_norm") or n.endswith("mix.norm"):
                 p.data.copy_(1.0 + 0.1 * torch.randn(p.shape, generator=g))
@@ -263,9 +529,27 @@ class HybridDecoder(nn.Module):
     def embed_tokens(self, input_ids, positions=None, scatter: bool = False):
         return ops.embedding(input_ids, self.embed)
 
+    def embed_step(self, input_ids: torch.Tensor, st: StepTensors, prev_tokens: Optional[torch.Tensor]) -> torch.Tensor:
+        """Sandwich designs: token ids of a batch plan -> the fp32 stream ahead of the first layer (the embedding's
+        bigram part reads and replaces the rows' previous tokens in `prev_tokens`)."""
+        big = self.cfg.bigram or {}
+        return sandwich.embed_bigram_norm(input_ids, self.embed, self.bigram, int(big.get("mul_prev", 0)),
+                                          int(big.get("mul_cur", 0)), self.embed_norm, self.embed_norm_bias,
+                                          float(self.cfg.rms_norm_eps), st.cu_q, st.first_pos, st.state_slots,
+                                          prev_tokens)
+
     # ------------------------------------------------------------------------- checkpoint names
     def checkpoint_tensors(self) -> Dict[str, torch.Tensor]:
         """Checkpoint name -> the view of this model's parameters that holds it (fused projections are sliced)."""
+        if self.sandwich:
+            out = {"embed": self.embed.data, "head": self.head.data, "final.norm": self.norm.data,
+                   "final.norm.b": self.norm_bias.data, "embed.norm": self.embed_norm.data,
+                   "embed.norm.b": self.embed_norm_bias.data}
+            if self.bigram is not None:
+                out["bigram"] = self.bigram.data
+            for i, blk in enumerate(self.layers):
+                out.update(blk.checkpoint_tensors(f"l{i}."))
+            return out
         out: Dict[str, torch.Tensor] = {"embed": self.embed.data, "head": self.head.data,
                                         "final.norm": self.norm.data.view(())}
         for i, blk in enumerate(self.layers):

@@ -181,6 +181,28 @@ def grouped_gemm_offsets(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor
     return _launch(x.contiguous(), w, offsets)
 
 
+def grouped_gemm_rows(x: torch.Tensor, w: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
+    """Forward-only grouped GEMM for ANY operand shape and for bf16 or fp32 (fp32: true fp32 products): the MFMA
+    kernel where it applies, otherwise an LDS-tiled kernel with fp32 accumulation. x [T, K] rows sorted by expert,
+    w [E, N, K], offsets int32 [>= E + 1] on the device. No host synchronisation on the GPU."""
+    E, N, K = w.shape
+    offsets = offsets[:E + 1]
+    if x.shape[0] == 0:
+        return x.new_zeros(0, N)
+    if grouped_gemm_offsets_ok(x, w):
+        return _launch(x.contiguous(), w, offsets)
+    if L.use_hip(x):
+        x = x.contiguous()
+        assert w.is_contiguous() and w.dtype == x.dtype and offsets.dtype == torch.int32 and x.shape[1] == K
+        out = torch.empty(x.shape[0], N, dtype=x.dtype, device=x.device)
+        L.check(L.lib().areal_grouped_gemm_plain(L.ptr(x), L.ptr(w), L.ptr(out), L.ptr(offsets), L.c_int(x.shape[0]),
+                                                 L.c_int(E), L.c_int(N), L.c_int(K), L.c_int(L.dtype_flag(x)),
+                                                 L.stream_ptr()), "grouped_gemm_plain")
+        return out
+    off = offsets.tolist()
+    return grouped_gemm_ref(x, w, [off[e + 1] - off[e] for e in range(E)])
+
+
 def grouped_gemm(x: torch.Tensor, w: torch.Tensor, counts: List[int]) -> torch.Tensor:
     """x [T, K] rows sorted by expert, w [E, N, K], counts[e] rows per expert (host ints, sum = T)."""
     if _hip_ok(x, w) and x.shape[0] > 0 and _prefer_library(x.shape[0], w.shape[0]):

@@ -149,3 +149,37 @@ def moe_sort(flat_e: torch.Tensor, n_experts: int, k: int):
 def moe_combine(ys: torch.Tensor, w: torch.Tensor, order: torch.Tensor, inv: torch.Tensor) -> torch.Tensor:
     """Expert outputs in expert order ys [T*k, H], routing weights w [T, k] -> [T, H]."""
     return _CombineFn.apply(ys, w, order, inv)
+
+
+def clamped_glu(gu: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """Gated unit with clamped pre-activations: gu [n, 2F] = gate | up ->  g sigmoid(alpha g) (u + 1)  with
+    g = min(gate, limit), u = clamp(up, -limit, limit); [n, F] in gu's dtype (fp32 arithmetic)."""
+    n, F2 = gu.shape
+    F = F2 // 2
+    if L.use_hip(gu):
+        assert gu.is_contiguous()
+        out = torch.empty(n, F, dtype=gu.dtype, device=gu.device)
+        if n:
+            L.check(L.lib().areal_clamped_glu(L.ptr(gu), L.ptr(out), L.c_int64(n), L.c_int(F), L.c_float(limit),
+                                              L.c_float(alpha), L.c_int(L.dtype_flag(gu)), L.stream_ptr()),
+                    "clamped_glu")
+        return out
+    g = gu[:, :F].float().clamp(max=limit)
+    u = gu[:, F:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def combine_rows_w32(ys: torch.Tensor, inv: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """out[t] = sum_j w[t, j] * ys[inv[t*k + j]] with fp32 weights w [T, k] and an fp32 sum; ys [T*k, H] in expert
+    order, result in ys's dtype."""
+    T, k = w.shape
+    assert w.dtype == torch.float32
+    if L.use_hip(ys):
+        ys = ys.contiguous()
+        out = torch.empty(T, ys.shape[1], dtype=ys.dtype, device=ys.device)
+        if T:
+            L.check(L.lib().areal_moe_combine_w32(L.ptr(ys), L.ptr(inv), L.ptr(w.contiguous()), L.ptr(out),
+                                                  L.c_int64(T), L.c_int(k), L.c_int(ys.shape[1]),
+                                                  L.c_int(L.dtype_flag(ys)), L.stream_ptr()), "moe_combine_w32")
+        return out
+    return (ys[inv].view(T, k, -1).float() * w.view(T, k, 1)).sum(1).to(ys.dtype)

@@ -41,6 +41,14 @@ def _run(cmd):
     return r
 
 
+def linked_sources() -> set:
+    """Stems of the sources the kernel library in the tree was linked from (empty: no library, or an unknown one)."""
+    manifest = BUILD_DIR / "libareal_hip.objs"
+    if not (OUT_DIR / "libareal_hip.so").exists() or not manifest.exists():
+        return set()
+    return {Path(n).stem for n in manifest.read_text().split()}
+
+
 def build_hip(verbose=True, only=None) -> Path:
     """`only`: stems of the sources to build the library from (a program that needs a few kernels of a fresh
     checkout); the next full build relinks it from everything."""

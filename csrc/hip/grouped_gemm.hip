@@ -454,3 +454,74 @@ extern "C" int areal_grouped_gemm_wgrad(const void* dy, const void* x, void* dw,
 #undef AREAL_GG_WGRAD
   return (int)hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Grouped product for ANY operand shape and for bf16 or fp32 storage (fp32: true fp32 multiply-adds): what the
+// matrix-core kernel above does not take (sizes that are no multiples of 64, fp32 serving). Workgroup (e, c) owns
+// expert e and 64 output columns and walks the expert's rows in tiles of 32; operands pass through LDS in k-chunks of
+// 32, every thread keeps 8 rows of one column. Row ranges come from the device, so the launch depends on shapes only.
+namespace {
+template <typename T> DEVINL float gg_ld(const T* p, size_t i);
+template <> DEVINL float gg_ld<bf16_t>(const bf16_t* p, size_t i) { return bf2f(p[i]); }
+template <> DEVINL float gg_ld<float>(const float* p, size_t i) { return p[i]; }
+template <typename T> DEVINL void gg_st(T* p, size_t i, float v);
+template <> DEVINL void gg_st<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f2bf(v); }
+template <> DEVINL void gg_st<float>(float* p, size_t i, float v) { p[i] = v; }
+
+template <typename T>
+__global__ void __launch_bounds__(256) grouped_gemm_plain_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                 T* __restrict__ out, const int* __restrict__ offsets,
+                                                                 int N, int K) {
+  __shared__ float xs[32][33];
+  __shared__ float ws[64][33];
+  const int e = blockIdx.x, n0 = blockIdx.y * 64, tid = threadIdx.x;
+  const int col = tid & 63, rg = tid >> 6;
+  const int r_lo = offsets[e], r_hi = offsets[e + 1];
+  const T* we = w + (size_t)e * N * K;
+  for (int r0 = r_lo; r0 < r_hi; r0 += 32) {
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += 32) {
+      __syncthreads();
+      for (int i = tid; i < 32 * 32; i += 256) {
+        const int r = i >> 5, kk = i & 31;
+        xs[r][kk] = (r0 + r < r_hi && k0 + kk < K) ? gg_ld<T>(x, (size_t)(r0 + r) * K + k0 + kk) : 0.f;
+      }
+      for (int i = tid; i < 64 * 32; i += 256) {
+        const int c = i >> 5, kk = i & 31;
+        ws[c][kk] = (n0 + c < N && k0 + kk < K) ? gg_ld<T>(we, (size_t)(n0 + c) * K + k0 + kk) : 0.f;
+      }
+      __syncthreads();
+#pragma unroll 8
+      for (int kk = 0; kk < 32; ++kk) {
+        const float wv = ws[col][kk];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += xs[rg * 8 + i][kk] * wv;
+      }
+    }
+    if (n0 + col < N) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int r = r0 + rg * 8 + i;
+        if (r < r_hi) gg_st<T>(out, (size_t)r * N + n0 + col, acc[i]);
+      }
+    }
+  }
+}
+}  // namespace
+
+// x [T, K] rows sorted by expert, w [E, N, K] contiguous, offsets [E + 1] on the device; dt 0: bf16, 1: fp32.
+extern "C" int areal_grouped_gemm_plain(const void* x, const void* w, void* out, const int* offsets, int T, int E,
+                                        int N, int K, int dt, hipStream_t st) {
+  if (T == 0 || E == 0) return 0;
+  if (N < 1 || K < 1 || E > 65535 * 32) return -1;
+  const dim3 grid(E, (N + 63) / 64);
+  if (dt == 0)
+    hipLaunchKernelGGL(grouped_gemm_plain_kernel<bf16_t>, grid, dim3(256), 0, st, (const bf16_t*)x, (const bf16_t*)w,
+                       (bf16_t*)out, offsets, N, K);
+  else
+    hipLaunchKernelGGL(grouped_gemm_plain_kernel<float>, grid, dim3(256), 0, st, (const float*)x, (const float*)w,
+                       (float*)out, offsets, N, K);
+  return (int)hipGetLastError();
+}

@@ -1,0 +1,321 @@
+// Attention through a shared low-rank latent over a paged cache of [c | r] rows (c: R latent numbers, r: P rotary
+// key numbers shared by all heads; token-major pages of 32).
+//
+//   latent_prep   per token: RMS norm (times weight) of the query latent -> cq, of the key/value latent -> cache c;
+//                 the rotary key part rotated at the token's position -> cache r
+//   latent_attn   s_h(i, j) = scale * (q~_h(i) . c(j) + rot_i(q^r_h(i)) . r(j)),  visible: 0 <= i - j < window
+//                 o~_h(i)   = sum_j softmax_j(s_h(i, .)) c(j)   [* sigmoid(gate_h(i))]
+//                 q~ are the queries already carried into latent space (absorbed key expansion); the rotary query
+//                 part arrives unrotated (the last P entries of every head of q) and is rotated here.
+//
+// All heads read the same keys, and the values are the first R entries of the keys: a workgroup owns a tile of BQ
+// queries x a group of HG heads, stages each 32-key page ONCE in LDS and uses it for both products. Scores, weights
+// and the accumulation are fp32 whatever the storage type T (bf16 / fp32).
+//
+// The same kernel serves prompt portions (grid x = query tiles x head groups, y = rows of the batch) and decoding
+// (BQ = 1, grid z = splits of the visible key range whose partial results `latent_attn_combine` merges).
+// Queries of row b are the LAST cu_q[b+1] - cu_q[b] positions of its context of ctx_len[b] tokens.
+// Rotation: pairs (i, i + P/2); table [n_pos][P] = cos | sin of position * frequency.
+#include "common.hpp"
+
+namespace {
+
+constexpr int PAGE = 32;
+
+template <typename T> DEVINL float ldf(const T* p, size_t i);
+template <> DEVINL float ldf<bf16_t>(const bf16_t* p, size_t i) { return bf2f(p[i]); }
+template <> DEVINL float ldf<float>(const float* p, size_t i) { return p[i]; }
+template <typename T> DEVINL void stf(T* p, size_t i, float v);
+template <> DEVINL void stf<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f2bf(v); }
+template <> DEVINL void stf<float>(float* p, size_t i, float v) { p[i] = v; }
+
+// One workgroup per token; wave 0: query latent, wave 1: key/value latent, wave 2: rotary key part.
+template <typename T>
+__global__ void __launch_bounds__(256) latent_prep_kernel(
+    const T* __restrict__ proj, int64_t row_stride, const T* __restrict__ qw, const T* __restrict__ cw,
+    const int* __restrict__ positions, const int64_t* __restrict__ slots, const float* __restrict__ table, int n_pos,
+    T* __restrict__ cq, T* __restrict__ cache, int Q, int R, int P, float eps) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* row = proj + (size_t)t * row_stride;
+  const int64_t slot = slots[t];
+  T* dst = slot >= 0 ? cache + (size_t)slot * (R + P) : nullptr;  // slot = page * 32 + offset
+  if (wave == 0) {
+    float ss = 0.f;
+    for (int i = lane; i < Q; i += 64) {
+      const float x = ldf<T>(row, i);
+      ss += x * x;
+    }
+    const float r = 1.f / sqrtf(wave_sum(ss) / (float)Q + eps);
+    for (int i = lane; i < Q; i += 64) stf<T>(cq, (size_t)t * Q + i, ldf<T>(row, i) * r * ldf<T>(qw, i));
+  } else if (wave == 1) {
+    if (!dst) return;
+    float ss = 0.f;
+    for (int i = lane; i < R; i += 64) {
+      const float x = ldf<T>(row, Q + i);
+      ss += x * x;
+    }
+    const float r = 1.f / sqrtf(wave_sum(ss) / (float)R + eps);
+    for (int i = lane; i < R; i += 64) stf<T>(dst, i, ldf<T>(row, Q + i) * r * ldf<T>(cw, i));
+  } else if (wave == 2) {
+    if (!dst) return;
+    const int pos = min(max(positions[t], 0), n_pos - 1);
+    const float* cs = table + (size_t)pos * P;
+    const int half = P / 2;
+    for (int i = lane; i < half; i += 64) {
+      const float u = ldf<T>(row, Q + R + i), v = ldf<T>(row, Q + R + half + i);
+      const float c = cs[i], s = cs[half + i];
+      stf<T>(dst, R + i, u * c - v * s);
+      stf<T>(dst, R + half + i, v * c + u * s);
+    }
+  }
+}
+
+struct LatentShape {
+  int H, HG, D, P, R, BQ;
+  __host__ __device__ int rows() const { return HG * BQ; }
+  __host__ __device__ int ks() const { return R + P + 1; }  // padded key row: conflict-free column walks
+  __host__ __device__ size_t floats() const {
+    return (size_t)rows() * (R + P) + (size_t)rows() * R + (size_t)rows() * PAGE + (size_t)PAGE * ks() + 3 * (size_t)rows();
+  }
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) latent_attn_kernel(
+    const T* __restrict__ q, const T* __restrict__ q_lat, const T* __restrict__ cache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, const T* __restrict__ gate,
+    int64_t gate_stride, T* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    LatentShape sh, float scale, int window, int nsplit) {
+  extern __shared__ float lds[];
+  const int H = sh.H, HG = sh.HG, D = sh.D, P = sh.P, R = sh.R, BQ = sh.BQ, KW = R + P, KS = sh.ks();
+  const int tid = threadIdx.x;
+  const int n_groups = (H + HG - 1) / HG;
+  const int tile = blockIdx.x / n_groups, h0 = (blockIdx.x % n_groups) * HG;
+  const int nh = min(HG, H - h0);
+  const int b = blockIdx.y, split = blockIdx.z;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
+  const int t0 = tile * BQ;
+  if (t0 >= qlen) return;
+  const int nq = min(BQ, qlen - t0);
+  const int ctx = ctx_len[b];
+  const int pos0 = ctx - qlen + t0;  // position of the tile's first query
+  const int NR = HG * BQ;            // (head, query) rows: r = hh * BQ + qi
+  float* qs = lds;                        // [NR][KW]
+  float* acc = qs + (size_t)NR * KW;      // [NR][R]
+  float* S = acc + (size_t)NR * R;        // [NR][32]
+  float* Kt = S + (size_t)NR * PAGE;      // [32][KS]
+  float* mrow = Kt + (size_t)PAGE * KS;   // [NR]
+  float* lrow = mrow + NR;
+  float* corr = lrow + NR;
+
+  const int half = P / 2;
+  for (int i = tid; i < NR * KW; i += 256) {
+    const int d = i % KW, r = i / KW, qi = r % BQ, hh = r / BQ;
+    float v = 0.f;
+    if (qi < nq && hh < nh) {
+      const size_t tok = (size_t)(q0 + t0 + qi);
+      if (d < R) {
+        v = ldf<T>(q_lat, (tok * H + h0 + hh) * R + d);
+      } else {
+        const int e = d - R, pi = e < half ? e : e - half;
+        const T* qr = q + (tok * H + h0 + hh) * (D + P) + D;
+        const float* cs = table + (size_t)min(max(pos0 + qi, 0), n_pos - 1) * P;
+        const float u = ldf<T>(qr, pi), w = ldf<T>(qr, half + pi), c = cs[pi], s = cs[half + pi];
+        v = e < half ? u * c - w * s : w * c + u * s;
+      }
+    }
+    qs[i] = v;
+  }
+  for (int i = tid; i < NR * R; i += 256) acc[i] = 0.f;
+  for (int i = tid; i < NR; i += 256) {
+    mrow[i] = -1e30f;
+    lrow[i] = 0.f;
+  }
+
+  // visible keys of the tile: [j_lo, j_hi); pages [p_lo, p_hi), this split's share of them
+  const int j_hi = pos0 + nq;
+  const int j_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int p_lo = j_lo / PAGE, p_hi = (j_hi + PAGE - 1) / PAGE;
+  const int per = (p_hi - p_lo + nsplit - 1) / nsplit;
+  const int my_lo = p_lo + split * per, my_hi = min(p_hi, my_lo + per);
+
+  for (int pg = my_lo; pg < my_hi; ++pg) {
+    const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
+    const int jb = pg * PAGE;
+    __syncthreads();  // Kt free (and, at the first page, the tile set-up visible)
+    const T* kp = cache + page * PAGE * KW;
+    if (sizeof(T) == 2 && KW % 8 == 0) {  // 16-byte loads
+      for (int i = tid; i < PAGE * KW / 8; i += 256) {
+        const int key = (8 * i) / KW;
+        const bf16x8 x = ld8(reinterpret_cast<const bf16_t*>(kp) + 8 * i);
+        float* dst = Kt + key * KS + (8 * i) % KW;
+        const bool live = jb + key < j_hi;  // rows past the last key may hold anything
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[e] = live ? bf2f(x[e]) : 0.f;
+      }
+    } else {
+      for (int i = tid; i < PAGE * KW; i += 256)
+        Kt[(i / KW) * KS + i % KW] = (jb + i / KW < j_hi) ? ldf<T>(kp, i) : 0.f;
+    }
+    __syncthreads();
+    // ---- scores
+    for (int e = tid; e < NR * PAGE; e += 256) {
+      const int kj = e % PAGE, r = e / PAGE, qi = r % BQ, hh = r / BQ;
+      const float* qv = qs + (size_t)r * KW;
+      const float* kv = Kt + kj * KS;
+      float s = 0.f;
+      for (int d = 0; d < KW; ++d) s += qv[d] * kv[d];
+      const int dist = pos0 + qi - (jb + kj);
+      const bool ok = qi < nq && hh < nh && dist >= 0 && (window <= 0 || dist < window);
+      S[e] = ok ? s * scale : -INFINITY;
+    }
+    __syncthreads();
+    // ---- running maximum / denominator per (head, query) row: 32 lanes a row
+    for (int r = tid >> 5; r < NR; r += 8) {
+      const float s = S[(size_t)r * PAGE + (tid & 31)];
+      float mx = s;
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+      const float m_old = mrow[r], m_new = fmaxf(m_old, mx);
+      const float p = expf(s - m_new);
+      float sum = p;
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+      S[(size_t)r * PAGE + (tid & 31)] = p;
+      if ((tid & 31) == 0) {
+        corr[r] = expf(m_old - m_new);
+        lrow[r] = lrow[r] * corr[r] + sum;
+        mrow[r] = m_new;
+      }
+    }
+    __syncthreads();
+    // ---- weights x latents (the first R entries of the staged keys)
+    for (int o = tid; o < NR * R; o += 256) {
+      const int v = o % R, r = o / R;
+      const float* pw = S + (size_t)r * PAGE;
+      float a = acc[o] * corr[r];
+#pragma unroll 8
+      for (int kj = 0; kj < PAGE; ++kj) a += pw[kj] * Kt[kj * KS + v];
+      acc[o] = a;
+    }
+  }
+  __syncthreads();
+  for (int o = tid; o < NR * R; o += 256) {
+    const int v = o % R, r = o / R, qi = r % BQ, hh = r / BQ;
+    if (qi >= nq || hh >= nh) continue;
+    const size_t tok = (size_t)(q0 + t0 + qi);
+    const int h = h0 + hh;
+    if (nsplit == 1) {
+      const float l = lrow[r];
+      float val = l > 0.f ? acc[o] / l : 0.f;
+      if (gate) val /= 1.f + expf(-ldf<T>(gate, tok * gate_stride + h));
+      stf<T>(out, (tok * H + h) * R + v, val);
+    } else {
+      part_acc[((tok * nsplit + split) * H + h) * R + v] = acc[o];
+      if (v == 0) {
+        part_ml[((tok * nsplit + split) * H + h) * 2] = mrow[r];
+        part_ml[((tok * nsplit + split) * H + h) * 2 + 1] = lrow[r];
+      }
+    }
+  }
+}
+
+// Merge of the key-range splits of one (token, head): grid (T, H).
+template <typename T>
+__global__ void __launch_bounds__(128) latent_attn_combine_kernel(const float* __restrict__ part_acc,
+                                                                  const float* __restrict__ part_ml,
+                                                                  const T* __restrict__ gate, int64_t gate_stride,
+                                                                  T* __restrict__ out, int H, int R, int nsplit) {
+  const size_t tok = blockIdx.x;
+  const int h = blockIdx.y;
+  float m = -1e30f;
+  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, part_ml[((tok * nsplit + s) * H + h) * 2]);
+  float l = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float* ml = part_ml + ((tok * nsplit + s) * H + h) * 2;
+    l += ml[1] * expf(ml[0] - m);
+  }
+  float g = 1.f;
+  if (gate) g = 1.f / (1.f + expf(-ldf<T>(gate, tok * gate_stride + h)));
+  const float inv = l > 0.f ? g / l : 0.f;
+  for (int v = threadIdx.x; v < R; v += 128) {
+    float a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float w = expf(part_ml[((tok * nsplit + s) * H + h) * 2] - m);
+      a += w * part_acc[((tok * nsplit + s) * H + h) * R + v];
+    }
+    stf<T>(out, (tok * H + h) * R + v, a * inv);
+  }
+}
+
+// Query tile and head group of a launch: the largest tile (up to `want` queries) x group that fits the LDS limit,
+// preferring whole-head launches (the staged keys are shared by all heads of the group).
+bool pick_shape(int H, int D, int P, int R, int want, LatentShape* out) {
+  for (int hg = H; hg >= 1; hg = (hg + 1) / 2) {
+    for (int bq = want; bq >= 1; bq >>= 1) {
+      LatentShape sh{H, hg, D, P, R, bq};
+      if (sh.floats() * sizeof(float) <= 156 * 1024) {
+        *out = sh;
+        return true;
+      }
+    }
+    if (hg == 1) break;
+  }
+  return false;
+}
+
+}  // namespace
+
+extern "C" int areal_latent_prep(const void* proj, int64_t row_stride, const void* qw, const void* cw,
+                                 const int* positions, const int64_t* slots, const float* table, int n_pos, void* cq,
+                                 void* cache, int T, int Q, int R, int P, float eps, int dt, hipStream_t st) {
+  if (T == 0) return 0;
+  if (P % 2 || n_pos < 1) return -1;
+  if (dt == 0)
+    hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(T), dim3(256), 0, st, (const bf16_t*)proj, row_stride,
+                       (const bf16_t*)qw, (const bf16_t*)cw, positions, slots, table, n_pos, (bf16_t*)cq,
+                       (bf16_t*)cache, Q, R, P, eps);
+  else
+    hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(T), dim3(256), 0, st, (const float*)proj, row_stride,
+                       (const float*)qw, (const float*)cw, positions, slots, table, n_pos, (float*)cq, (float*)cache,
+                       Q, R, P, eps);
+  return (int)hipGetLastError();
+}
+
+// B rows; row b's queries are tokens cu_q[b] .. cu_q[b+1]; max_q = longest row. nsplit > 1 needs part_acc
+// [T, nsplit, H, R] and part_ml [T, nsplit, H, 2] (fp32) and is meant for single-query rows.
+extern "C" int areal_latent_attn(const void* q, const void* q_lat, const void* cache, const int* block_tables,
+                                 int max_pages, const int* cu_q, const int* ctx_len, const float* table, int n_pos,
+                                 const void* gate, int64_t gate_stride, void* out, float* part_acc, float* part_ml,
+                                 int B, int max_q, int T, int H, int D, int P, int R, float scale, int window,
+                                 int nsplit, int dt, hipStream_t st) {
+  if (B == 0 || T == 0) return 0;
+  if (H < 1 || R < 1 || P % 2 || nsplit < 1 || n_pos < 1) return -1;
+  int want = 1;
+  while (want < 8 && want < max_q) want <<= 1;
+  LatentShape sh;
+  if (!pick_shape(H, D, P, R, want, &sh)) return -2;
+  const size_t lds = sh.floats() * sizeof(float);
+  if (nsplit > 1 && (!part_acc || !part_ml)) return -3;
+  const int n_groups = (H + sh.HG - 1) / sh.HG;
+  const dim3 grid(((max_q + sh.BQ - 1) / sh.BQ) * n_groups, B, nsplit);
+#define LAUNCH(TT)                                                                                                  \
+  do {                                                                                                              \
+    static size_t allowed = 64 * 1024; /* raised once: no attribute call inside a stream capture */                 \
+    if (lds > allowed) {                                                                                            \
+      HIP_RET(hipFuncSetAttribute((const void*)latent_attn_kernel<TT>, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                  160 * 1024));                                                                     \
+      allowed = 160 * 1024;                                                                                         \
+    }                                                                                                               \
+    hipLaunchKernelGGL(latent_attn_kernel<TT>, grid, dim3(256), lds, st, (const TT*)q, (const TT*)q_lat,            \
+                       (const TT*)cache, block_tables, max_pages, cu_q, ctx_len, table, n_pos, (const TT*)gate,     \
+                       gate_stride, (TT*)out, part_acc, part_ml, sh, scale, window, nsplit);                        \
+    if (nsplit > 1)                                                                                                 \
+      hipLaunchKernelGGL(latent_attn_combine_kernel<TT>, dim3(T, H), dim3(128), 0, st, part_acc, part_ml,           \
+                         (const TT*)gate, gate_stride, (TT*)out, H, R, nsplit);                                     \
+  } while (0)
+  if (dt == 0) LAUNCH(bf16_t);
+  else LAUNCH(float);
+#undef LAUNCH
+  return (int)hipGetLastError();
+}

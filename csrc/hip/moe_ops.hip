@@ -417,3 +417,70 @@ extern "C" int areal_moe_sort(const int64_t* flat_e, int64_t n, int bins, int k,
                      inv, src_row);
   return (int)hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// Gated unit with clamped pre-activations and the weighted recombination with fp32 routing weights, for bf16 or fp32
+// storage (dt 0 / 1):
+//   clamped_glu   gu [n, 2F] = gate | up  ->  g sigmoid(alpha g) (u + 1),  g = min(gate, limit), u = clamp(up, -limit, limit)
+//   combine_w32   out[t] = sum_j w[t, j] * src[inv[t k + j]]   (w fp32, the sum in fp32)
+namespace {
+template <typename T> DEVINL float mo_ld(const T* p, size_t i);
+template <> DEVINL float mo_ld<bf16_t>(const bf16_t* p, size_t i) { return bf2f(p[i]); }
+template <> DEVINL float mo_ld<float>(const float* p, size_t i) { return p[i]; }
+template <typename T> DEVINL void mo_st(T* p, size_t i, float v);
+template <> DEVINL void mo_st<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f2bf(v); }
+template <> DEVINL void mo_st<float>(float* p, size_t i, float v) { p[i] = v; }
+
+template <typename T>
+__global__ void __launch_bounds__(256) clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t n,
+                                                          int F, float limit, float alpha) {
+  const int64_t total = n * (int64_t)F;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / F;
+    const int c = (int)(i - r * F);
+    const float g = fminf(mo_ld<T>(gu, (size_t)r * 2 * F + c), limit);
+    const float u = fminf(fmaxf(mo_ld<T>(gu, (size_t)r * 2 * F + F + c), -limit), limit);
+    mo_st<T>(out, (size_t)i, g / (1.f + expf(-alpha * g)) * (u + 1.f));
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) moe_combine_w32_kernel(const T* __restrict__ src,
+                                                              const int64_t* __restrict__ inv,
+                                                              const float* __restrict__ w, T* __restrict__ out, int k,
+                                                              int H) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < H; c += 256) {
+    float a = 0.f;
+    for (int j = 0; j < k; ++j) a += w[t * k + j] * mo_ld<T>(src, (size_t)inv[t * k + j] * H + c);
+    mo_st<T>(out, (size_t)t * H + c, a);
+  }
+}
+}  // namespace
+
+extern "C" int areal_clamped_glu(const void* gu, void* out, int64_t n, int F, float limit, float alpha, int dt,
+                                 hipStream_t st) {
+  if (n == 0 || F == 0) return 0;
+  const int64_t total = n * (int64_t)F;
+  const unsigned blocks = (unsigned)((total + 255) / 256 < 65535 * 16 ? (total + 255) / 256 : 65535 * 16);
+  if (dt == 0)
+    hipLaunchKernelGGL(clamped_glu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, st, (const bf16_t*)gu, (bf16_t*)out, n,
+                       F, limit, alpha);
+  else
+    hipLaunchKernelGGL(clamped_glu_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float*)gu, (float*)out, n, F,
+                       limit, alpha);
+  return (int)hipGetLastError();
+}
+
+extern "C" int areal_moe_combine_w32(const void* src, const int64_t* inv, const float* w, void* out, int64_t T, int k,
+                                     int H, int dt, hipStream_t st) {
+  if (T == 0) return 0;
+  if (k < 1) return -3;
+  if (dt == 0)
+    hipLaunchKernelGGL(moe_combine_w32_kernel<bf16_t>, dim3((unsigned)T), dim3(256), 0, st, (const bf16_t*)src, inv, w,
+                       (bf16_t*)out, k, H);
+  else
+    hipLaunchKernelGGL(moe_combine_w32_kernel<float>, dim3((unsigned)T), dim3(256), 0, st, (const float*)src, inv, w,
+                       (float*)out, k, H);
+  return (int)hipGetLastError();
+}
