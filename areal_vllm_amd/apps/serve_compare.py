@@ -5,6 +5,10 @@ transformer (grouped-query attention with q/k norm, gated MLP) of the same width
 the width of its MLP - parameter count are served by the rollout engine on random weights: the same prompts, the same
 number of new tokens, prefill plans and captured decode graphs. Reported per model: prompt tokens/s over the prefill
 plans and generated tokens/s over the decode plans (the engine's own clocks), and the parameters per token.
+
+The Lufivik design (latent attention with a sliding window, routed clamped-GLU experts, sublayers between two layer
+norms) is compared the same way with a Qwen3-MoE-style transformer: the same width, depth, heads, experts and experts
+per token, its experts as wide as the parameter budget allows.
 """
 import json
 import sys
@@ -18,6 +22,13 @@ SIZES = {
     "w1024": (1024, 6, 8, 2, 128, 4096, 512),
     "w2048": (2048, 6, 16, 4, 128, 8192, 512),
     "w4096": (4096, 3, 32, 8, 128, 14336, 1024),
+}
+# Lufivik: width, layers, heads, unrotated / rotary / value size per head, query / key-value latent size, window,
+# experts, experts per token, expert width
+LUFIVIK_SIZES = {
+    "w1024": (1024, 4, 8, 64, 32, 64, 384, 256, 512, 16, 2, 512),
+    "w2048": (2048, 4, 16, 128, 64, 128, 768, 512, 1024, 32, 4, 768),
+    "w4096": (4096, 2, 32, 128, 64, 128, 1536, 512, 1024, 64, 4, 1024),
 }
 VOCAB = 32768
 
@@ -35,6 +46,31 @@ def kuzanex_dict(width, layers, heads, kv, dim, ff, window) -> Dict[str, Any]:
                        "mixer": {"heads": heads // 2, "dim": dim, "vdim": 2 * dim, "gate_cap": 12.0}})
     return {"architecture": "Kuzanex", "layers": ls, "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "vocab": VOCAB,
             "width": width}
+
+
+def lufivik_dict(width, layers, heads, dim, rot, vdim, q_rank, kv_rank, window, experts, top, ff) -> Dict[str, Any]:
+    layer = {"type": "latent_attention",
+             "mixer": {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+                       "scale": (dim + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot}, "mask": {"size": window}},
+             "mlp": {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}}
+    return {"architecture": "Lufivik", "layers": [json.loads(json.dumps(layer)) for _ in range(layers)],
+            "norm": {"eps": 1e-5}, "canon": {"taps": 4},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "vocab": VOCAB, "width": width}
+
+
+def moe_twin_config(lcfg, width, layers, heads, experts, top):
+    """Qwen3-MoE-style transformer (grouped-query attention, head size 128, routed SwiGLU experts) with the experts
+    as wide as the parameter budget of the Lufivik model allows."""
+    from ..models.config import ModelConfig
+
+    dim, kv = 128, max(1, heads // 4)
+    body = lcfg.n_params(with_embedding=False)
+    attn = width * (heads + 2 * kv) * dim + width * heads * dim
+    inter = max(64, int(round((body / layers - attn - width * experts) / (3 * width * experts) / 64)) * 64)
+    return ModelConfig(family="qwen3_moe", vocab_size=VOCAB, hidden_size=width, n_layers=layers, n_q_heads=heads,
+                       n_kv_heads=kv, head_dim=dim, intermediate_size=inter, moe_intermediate_size=inter,
+                       n_experts=experts, n_experts_per_tok=top, norm_topk_prob=True, tie_word_embeddings=False,
+                       qkv_bias=False, qk_norm=True, rope_theta=1e6, max_position_embeddings=8192, rms_norm_eps=1e-6)
 
 
 def twin_config(kcfg, width, layers, heads, kv, dim):
@@ -81,10 +117,32 @@ def measure(cfg, n_prompts: int, prompt_len: int, new_tokens: int, device) -> Di
     return out
 
 
-def run(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, device="cuda") -> int:
+def run_lufivik(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, dev) -> int:
+    from ..models.config import ModelConfig
+
+    for name in sizes:
+        width, layers, heads, dim, rot, vdim, q_rank, kv_rank, window, experts, top, ff = LUFIVIK_SIZES[name]
+        lcfg = ModelConfig.from_hf_dict(lufivik_dict(*LUFIVIK_SIZES[name]))
+        tcfg = moe_twin_config(lcfg, width, layers, heads, experts, top)
+        row = {"design": "lufivik", "size": name, "width": width, "layers": layers, "heads": heads,
+               "kv_rank": kv_rank, "rot_dim": rot, "window": window, "experts": experts, "top": top, "expert_ff": ff,
+               "twin_expert_ff": tcfg.moe_intermediate_size, "prompts": n_prompts, "prompt_len": prompt_len,
+               "new_tokens": new_tokens, "dtype": "bf16", "data": "synthetic"}
+        for label, cfg in (("lufivik", lcfg), ("qwen3_moe_twin", tcfg)):
+            m = measure(cfg, n_prompts, prompt_len, new_tokens, dev)
+            row[label] = {"params_no_embedding": cfg.n_params(with_embedding=False), **{k: round(v, 1) for k, v in m.items()}}
+        row["prefill_ratio"] = round(row["lufivik"]["prefill_tok_s"] / row["qwen3_moe_twin"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row["lufivik"]["decode_tok_s"] / row["qwen3_moe_twin"]["decode_tok_s"], 3)
+        print(json.dumps(row), flush=True)
+    return 0
+
+
+def run(sizes: List[str], n_prompts: int, prompt_len: int, new_tokens: int, device="cuda", design="kuzanex") -> int:
     from ..models.config import ModelConfig
 
     dev = torch.device(device, 0) if device == "cuda" else torch.device(device)
+    if design == "lufivik":
+        return run_lufivik(sizes, n_prompts, prompt_len, new_tokens, dev)
     for name in sizes:
         width, layers, heads, kv, dim, ff, window = SIZES[name]
         kcfg = ModelConfig.from_hf_dict(kuzanex_dict(width, layers, heads, kv, dim, ff, window))

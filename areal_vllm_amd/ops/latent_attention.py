@@ -91,11 +91,13 @@ def decode_splits(batch: int, window: int, max_context: int) -> int:
 def latent_attention(q: torch.Tensor, q_lat: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
                      cu_q: torch.Tensor, ctx_len: torch.Tensor, max_q: int, dim: int, rot: int, scale: float,
                      window: int, table: torch.Tensor, gate: Optional[torch.Tensor] = None, nsplit: int = 1,
-                     workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+                     workspace: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                     matrix_cores: bool = True) -> torch.Tensor:
     """q [T, H, dim + rot] (its last `rot` entries per head are the UNROTATED rotary query part; the kernel rotates them
     at the query's position), q_lat [T, H, R] absorbed queries. Row b owns tokens cu_q[b]:cu_q[b+1], the LAST
     positions of its context of ctx_len[b] tokens, whose cache rows are written already. gate [T, H] (unit stride
-    along the heads) or None. Returns o~ [T, H, R] (times sigmoid(gate))."""
+    along the heads) or None. `matrix_cores`: bf16 rows of several queries with the common latent / rotary sizes run
+    the MFMA kernel (False: always the plain one). Returns o~ [T, H, R] (times sigmoid(gate))."""
     T, H, R = q_lat.shape
     B = cu_q.numel() - 1
     assert q.shape == (T, H, dim + rot) and cache.shape[2] == R + rot and table.shape[1] == rot
@@ -118,7 +120,8 @@ def latent_attention(q: torch.Tensor, q_lat: torch.Tensor, cache: torch.Tensor, 
             L.ptr(ctx_len), L.ptr(table), L.c_int(table.shape[0]), L.ptr(gate),
             L.c_int64(gate.stride(0) if gate is not None else 0), L.ptr(out), L.ptr(pa), L.ptr(pm), L.c_int(B),
             L.c_int(int(max_q)), L.c_int(T), L.c_int(H), L.c_int(dim), L.c_int(rot), L.c_int(R), L.c_float(scale),
-            L.c_int(int(window)), L.c_int(int(nsplit)), L.c_int(L.dtype_flag(q)), L.stream_ptr()), "latent_attn")
+            L.c_int(int(window)), L.c_int(int(nsplit)), L.c_int(L.dtype_flag(q)), L.c_int(int(matrix_cores)),
+            L.stream_ptr()), "latent_attn")
         return out
     out = torch.zeros(T, H, R, dtype=torch.float32, device=q.device)
     cq, cl = cu_q.tolist(), ctx_len.tolist()

@@ -105,6 +105,9 @@ def parse_args():
                         "beside a Qwen3-style transformer of equal size, one JSON line per size; comma-separated names "
                         "out of w1024, w2048, w4096, or 'all' (--prompts-per-gpu prompts of --prompt-len-max tokens, "
                         "--max-new-tokens new tokens each)")
+    p.add_argument("--serve-compare-design", default="kuzanex", choices=["kuzanex", "lufivik"],
+                   help="the layer-list design --serve-compare measures: kuzanex beside a Qwen3-style twin, or lufivik "
+                        "(latent attention, routed experts) beside a Qwen3-MoE-style twin")
     a = p.parse_args()
     if a.seq_len:
         a.max_new_tokens = a.seq_len - a.prompt_len_max
@@ -281,7 +284,8 @@ def main():
         from areal_vllm_amd.apps import serve_compare
 
         names = list(serve_compare.SIZES) if args.serve_compare == "all" else args.serve_compare.split(",")
-        sys.exit(serve_compare.run(names, args.prompts_per_gpu, args.prompt_len_max, args.max_new_tokens, args.device))
+        sys.exit(serve_compare.run(names, args.prompts_per_gpu, args.prompt_len_max, args.max_new_tokens, args.device,
+                                   design=args.serve_compare_design))
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ and "RANK" not in os.environ:
         sys.exit(launch_ranks(args))
     run_rank(args)

@@ -220,6 +220,183 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------------------------------
+// Matrix-core version for bf16 prompt portions. One workgroup = 16 queries x a group of up to 8 heads, one head per
+// wave. Per 32-key page:
+//   stage   the page's [c | r] rows -> LDS KT [32][KW + 8] (bf16), and the latent part transposed -> VT [R][32 + 8]
+//   scores  q (registers: absorbed query | rotated rotary part, bf16) x KT^T, bf16 MFMA 16x16x32 with fp32
+//           accumulation; scale and mask in fp32; running maximum / denominator of the wave's 16 rows in registers
+//           (a row's keys sit in the 16 lanes of one quad); the weight p (fp32) goes into the wave's own LDS tile as
+//           the pair (bf16(p), bf16(p - bf16(p)))
+//   p.c     bf16 MFMA over the (hi, lo) pairs as 32 k-slots against the latent columns taken twice: the product
+//           carries 16 bits of p's mantissa (the latents themselves are bf16), fp32 accumulation in registers
+// KW32 = (R + P) / 32 k-steps of the scores, R16 = R / 16 output tiles.
+template <int KW32, int R16>
+__global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ q_lat, const bf16_t* __restrict__ cache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
+    const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, const bf16_t* __restrict__ gate,
+    int64_t gate_stride, bf16_t* __restrict__ out, int H, int HG, int D, float scale, int window) {
+  constexpr int KW = KW32 * 32, R = R16 * 16, P = KW - R, KS = KW + 8, VS = PAGE + 8, SS = PAGE + 4;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  bf16_t* KT = reinterpret_cast<bf16_t*>(smem);                  // [32][KS]
+  bf16_t* VT = KT + (size_t)PAGE * KS;                           // [R][VS]
+  unsigned* PM = reinterpret_cast<unsigned*>(VT + (size_t)R * VS);  // [waves][16][SS] 4-byte slots
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthr = blockDim.x;
+  const int r16 = lane & 15, quad = lane >> 4;
+  const int n_groups = (H + HG - 1) / HG;
+  const int tile = blockIdx.x / n_groups, h = (blockIdx.x % n_groups) * HG + wave;
+  const bool own = h < H;  // waves past the last head only help staging
+  const int b = blockIdx.y;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0, t0 = tile * 16;
+  if (t0 >= qlen) return;
+  const int nq = min(16, qlen - t0), ctx = ctx_len[b], pos0 = ctx - qlen + t0;
+  unsigned* pm = PM + (size_t)wave * 16 * SS;
+
+  bf16x8 qf[KW32];
+  f32x4 acc[R16];
+  float mrow[4], lrow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    mrow[i] = -1e30f;
+    lrow[i] = 0.f;
+  }
+#pragma unroll
+  for (int vt = 0; vt < R16; ++vt) acc[vt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ks = 0; ks < KW32; ++ks) {
+    qf[ks] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
+    if (own && r16 < nq) {
+      const size_t tok = (size_t)(q0 + t0 + r16);
+      const int d = 32 * ks + 8 * quad;
+      if (d < R) {
+        qf[ks] = ld8(q_lat + (tok * H + h) * R + d);
+      } else {  // rotary part: entry e pairs with e +- P/2
+        constexpr int half = P / 2;
+        const int e = d - R, pi = e < half ? e : e - half;
+        const bf16_t* qr = q + (tok * H + h) * (size_t)(D + P) + D;
+        const bf16x8 u = ld8(qr + pi), w = ld8(qr + half + pi);
+        const float* cs = table + (size_t)min(max(pos0 + r16, 0), n_pos - 1) * P;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float c = cs[pi + k], sn = cs[half + pi + k], uu = bf2f(u[k]), ww = bf2f(w[k]);
+          qf[ks][k] = f2bf(e < half ? uu * c - ww * sn : ww * c + uu * sn);
+        }
+      }
+    }
+  }
+  const int j_hi = pos0 + nq;
+  const int j_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int p_lo = j_lo / PAGE, p_hi = (j_hi + PAGE - 1) / PAGE;
+
+  for (int pg = p_lo; pg < p_hi; ++pg) {
+    const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
+    const int jb = pg * PAGE;
+    __syncthreads();  // the page before is consumed
+    const bf16_t* kp = cache + page * PAGE * KW;
+    for (int i = tid; i < PAGE * (KW / 8); i += nthr) {
+      const int dv = i % (KW / 8), key = i / (KW / 8);
+      bf16x8 x = ld8(kp + (size_t)key * KW + 8 * dv);
+      if (jb + key >= j_hi) x = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};  // rows past the last key may hold anything
+      st8(KT + (size_t)key * KS + 8 * dv, x);
+      if (8 * dv < R) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) VT[(size_t)(8 * dv + e) * VS + key] = x[e];
+      }
+    }
+    __syncthreads();
+    if (own) {
+      f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KW32; ++ks) {
+        const bf16x8 b0 = ld8(KT + (size_t)r16 * KS + 32 * ks + 8 * quad);
+        const bf16x8 b1 = ld8(KT + (size_t)(16 + r16) * KS + 32 * ks + 8 * quad);
+        c0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], b0, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], b1, c1, 0, 0, 0);
+      }
+      f32x4 cf;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int qi = 4 * quad + i;
+        const int d0 = pos0 + qi - (jb + r16), d1 = d0 - 16;
+        const bool ok0 = qi < nq && d0 >= 0 && (window <= 0 || d0 < window);
+        const bool ok1 = qi < nq && d1 >= 0 && (window <= 0 || d1 < window);
+        const float s0 = ok0 ? c0[i] * scale : -INFINITY, s1 = ok1 ? c1[i] * scale : -INFINITY;
+        float mx = fmaxf(s0, s1);
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float m_new = fmaxf(mrow[i], mx);
+        const float p0 = __expf(s0 - m_new), p1 = __expf(s1 - m_new);
+        float sum = p0 + p1;
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        cf[i] = __expf(mrow[i] - m_new);
+        lrow[i] = lrow[i] * cf[i] + sum;
+        mrow[i] = m_new;
+        const bf16_t h0 = f2bf(p0), h1 = f2bf(p1);
+        const bf16_t l0 = f2bf(p0 - bf2f(h0)), l1 = f2bf(p1 - bf2f(h1));
+        pm[qi * SS + r16] = (unsigned)__builtin_bit_cast(unsigned short, h0) |
+                            ((unsigned)__builtin_bit_cast(unsigned short, l0) << 16);
+        pm[qi * SS + 16 + r16] = (unsigned)__builtin_bit_cast(unsigned short, h1) |
+                                 ((unsigned)__builtin_bit_cast(unsigned short, l1) << 16);
+      }
+#pragma unroll
+      for (int vt = 0; vt < R16; ++vt) acc[vt] *= cf;
+    }
+    __syncthreads();  // the wave's weights are in its tile
+    if (own) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(pm + r16 * SS + 16 * kb + 4 * quad);
+#pragma unroll
+        for (int vt = 0; vt < R16; ++vt) {
+          const bf16x4 v4 = *reinterpret_cast<const bf16x4*>(VT + (size_t)(16 * vt + r16) * VS + 16 * kb + 4 * quad);
+          const bf16x8 bb = {v4[0], v4[0], v4[1], v4[1], v4[2], v4[2], v4[3], v4[3]};
+          acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bb, acc[vt], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (!own) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int qi = 4 * quad + i;
+    if (qi >= nq) continue;
+    const size_t tok = (size_t)(q0 + t0 + qi);
+    float f = lrow[i] > 0.f ? 1.f / lrow[i] : 0.f;
+    if (gate) f /= 1.f + expf(-bf2f(gate[tok * gate_stride + h]));
+#pragma unroll
+    for (int vt = 0; vt < R16; ++vt) out[(tok * H + h) * R + 16 * vt + r16] = f2bf(acc[vt][i] * f);
+  }
+}
+
+size_t mfma_lds_bytes(int R, int P, int waves) {
+  return (size_t)PAGE * (R + P + 8) * 2 + (size_t)R * (PAGE + 8) * 2 + (size_t)waves * 16 * (PAGE + 4) * 4;
+}
+
+// Shapes the matrix-core kernel is instantiated for: (latent size, rotary size), unrotated key size D.
+bool mfma_usable(int R, int P, int D) {
+  if (D % 8 != 0) return false;  // 16-byte loads of the rotary query part
+  return (R == 512 && P == 64) || (R == 256 && (P == 64 || P == 32)) || (R == 128 && (P == 64 || P == 32)) ||
+         (R == 64 && (P == 64 || P == 32));
+}
+
+template <int KW32, int R16>
+int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q, const bf16_t* q_lat,
+                const bf16_t* cache, const int* bt, int max_pages, const int* cu_q, const int* ctx_len,
+                const float* table, int n_pos, const bf16_t* gate, int64_t gate_stride, bf16_t* out, int H, int HG, int D,
+                float scale, int window) {
+  static bool raised = false;  // once per kernel: no attribute call inside a stream capture later
+  if (!raised) {
+    HIP_RET(hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<KW32, R16>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    raised = true;
+  }
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<KW32, R16>), grid, dim3(nthr), lds, st, q, q_lat, cache, bt, max_pages,
+                     cu_q, ctx_len, table, n_pos, gate, gate_stride, out, H, HG, D, scale, window);
+  return (int)hipGetLastError();
+}
+
 // Merge of the key-range splits of one (token, head): grid (T, H).
 template <typename T>
 __global__ void __launch_bounds__(128) latent_attn_combine_kernel(const float* __restrict__ part_acc,
@@ -288,9 +465,22 @@ extern "C" int areal_latent_attn(const void* q, const void* q_lat, const void* c
                                  int max_pages, const int* cu_q, const int* ctx_len, const float* table, int n_pos,
                                  const void* gate, int64_t gate_stride, void* out, float* part_acc, float* part_ml,
                                  int B, int max_q, int T, int H, int D, int P, int R, float scale, int window,
-                                 int nsplit, int dt, hipStream_t st) {
+                                 int nsplit, int dt, int matrix_cores, hipStream_t st) {
   if (B == 0 || T == 0) return 0;
   if (H < 1 || R < 1 || P % 2 || nsplit < 1 || n_pos < 1) return -1;
+  if (matrix_cores && dt == 0 && nsplit == 1 && max_q > 1 && mfma_usable(R, P, D)) {
+    const int hg = H < 8 ? H : 8, n_groups = (H + hg - 1) / hg;
+    const dim3 mgrid(((max_q + 15) / 16) * n_groups, B, 1);
+    const size_t mlds = mfma_lds_bytes(R, P, hg);
+#define MFMA_ARGS                                                                                                 \
+  mgrid, 64 * hg, mlds, st, (const bf16_t*)q, (const bf16_t*)q_lat, (const bf16_t*)cache, block_tables, max_pages, \
+      cu_q, ctx_len, table, n_pos, (const bf16_t*)gate, gate_stride, (bf16_t*)out, H, hg, D, scale, window
+    if (R == 512) return launch_mfma<18, 32>(MFMA_ARGS);
+    if (R == 256) return P == 64 ? launch_mfma<10, 16>(MFMA_ARGS) : launch_mfma<9, 16>(MFMA_ARGS);
+    if (R == 128) return P == 64 ? launch_mfma<6, 8>(MFMA_ARGS) : launch_mfma<5, 8>(MFMA_ARGS);
+    return P == 64 ? launch_mfma<4, 4>(MFMA_ARGS) : launch_mfma<3, 4>(MFMA_ARGS);
+#undef MFMA_ARGS
+  }
   int want = 1;
   while (want < 8 && want < max_q) want <<= 1;
   LatentShape sh;

@@ -173,7 +173,10 @@ def _mixer_cfg(H, D, P, V, R, window, scale=0.3, base=10000.0):
 @pytest.mark.parametrize("device,dtype", OP_CASES)
 @pytest.mark.parametrize("H,D,P,V,R,window", [(4, 16, 8, 24, 32, 37), (3, 8, 8, 8, 8, 32), (1, 40, 4, 16, 24, 5),
                                               (6, 32, 32, 32, 128, 40), (2, 64, 64, 128, 72, 0), (5, 24, 2, 8, 40, 1),
-                                              (16, 16, 16, 16, 64, 33)])
+                                              (16, 16, 16, 16, 64, 33),
+                                              # latent / rotary sizes the matrix-core kernel takes (bf16 prompt rows)
+                                              (16, 64, 64, 64, 512, 70), (9, 16, 32, 16, 256, 45), (3, 24, 64, 8, 64, 33),
+                                              (4, 8, 64, 24, 256, 0), (2, 12, 64, 16, 128, 31)])
 def test_latent_attention_edges_pages_portions_and_splits(device, dtype, H, D, P, V, R, window):
     """A key that dominates its query's scores sits just inside and just outside the window, on both sides of page
     borders, at position 0 and hundreds of tokens back; whole prompt, portions down to two tokens, several rows in
