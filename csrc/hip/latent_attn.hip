@@ -221,40 +221,60 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------------------------
-// Matrix-core version for bf16 prompt portions. One workgroup = 16 queries x a group of up to 8 heads, one head per
-// wave. Per 32-key page:
+// Matrix-core version for bf16. The 16 rows of a matrix-core tile are
+//   prompt portions (DEC = false): 16 queries of ONE head; a workgroup = 16 queries x a group of heads;
+//   decoding        (DEC = true):  the 16 heads of a head group of ONE query; grid z = splits of the key range.
+// RS waves share a tile's rows: each computes the scores (cheap beside p.c) and owns R / RS of the output columns,
+// which keeps the fp32 accumulators of large latents in registers. Per 32-key page:
 //   stage   the page's [c | r] rows -> LDS KT [32][KW + 8] (bf16), and the latent part transposed -> VT [R][32 + 8]
-//   scores  q (registers: absorbed query | rotated rotary part, bf16) x KT^T, bf16 MFMA 16x16x32 with fp32
-//           accumulation; scale and mask in fp32; running maximum / denominator of the wave's 16 rows in registers
-//           (a row's keys sit in the 16 lanes of one quad); the weight p (fp32) goes into the wave's own LDS tile as
-//           the pair (bf16(p), bf16(p - bf16(p)))
+//   scores  rows (registers: absorbed query | rotated rotary part, bf16) x KT^T, bf16 MFMA 16x16x32 with fp32
+//           accumulation; scale and mask in fp32; running maximum / denominator of the 16 rows in registers (a row's
+//           keys sit in the 16 lanes of one quad); the weight p (fp32) goes into the wave's own LDS tile as the pair
+//           (bf16(p), bf16(p - bf16(p)))
 //   p.c     bf16 MFMA over the (hi, lo) pairs as 32 k-slots against the latent columns taken twice: the product
 //           carries 16 bits of p's mantissa (the latents themselves are bf16), fp32 accumulation in registers
 // KW32 = (R + P) / 32 k-steps of the scores, R16 = R / 16 output tiles.
-template <int KW32, int R16>
+template <int KW32, int R16, int RS, bool DEC>
 __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ q_lat, const bf16_t* __restrict__ cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, const bf16_t* __restrict__ gate,
-    int64_t gate_stride, bf16_t* __restrict__ out, int H, int HG, int D, float scale, int window) {
-  constexpr int KW = KW32 * 32, R = R16 * 16, P = KW - R, KS = KW + 8, VS = PAGE + 8, SS = PAGE + 4;
+    int64_t gate_stride, bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, int H,
+    int HG, int D, float scale, int window, int nsplit) {
+  constexpr int KW = KW32 * 32, R = R16 * 16, P = KW - R, KS = KW + 8, VS = PAGE + 8, SS = PAGE + 4, NT = R16 / RS;
+  static_assert(R16 % RS == 0, "output tiles split evenly over the waves of a row tile");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16_t* KT = reinterpret_cast<bf16_t*>(smem);                  // [32][KS]
   bf16_t* VT = KT + (size_t)PAGE * KS;                           // [R][VS]
   unsigned* PM = reinterpret_cast<unsigned*>(VT + (size_t)R * VS);  // [waves][16][SS] 4-byte slots
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthr = blockDim.x;
   const int r16 = lane & 15, quad = lane >> 4;
-  const int n_groups = (H + HG - 1) / HG;
-  const int tile = blockIdx.x / n_groups, h = (blockIdx.x % n_groups) * HG + wave;
-  const bool own = h < H;  // waves past the last head only help staging
-  const int b = blockIdx.y;
-  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0, t0 = tile * 16;
-  if (t0 >= qlen) return;
-  const int nq = min(16, qlen - t0), ctx = ctx_len[b], pos0 = ctx - qlen + t0;
+  const int part = wave % RS, slot = wave / RS;
+  const int b = blockIdx.y, split = DEC ? blockIdx.z : 0;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0, ctx = ctx_len[b];
+  // rows of this wave's tile: (token, head) of row r, how many rows are real, position of row r's query
+  int t0, hbase, nrows, pos0;
+  if (DEC) {
+    if (qlen < 1) return;
+    t0 = 0;
+    hbase = blockIdx.x * 16;
+    nrows = min(16, H - hbase);
+    pos0 = ctx - 1;
+  } else {
+    const int n_groups = (H + HG - 1) / HG;
+    t0 = (blockIdx.x / n_groups) * 16;
+    if (t0 >= qlen) return;
+    hbase = (blockIdx.x % n_groups) * HG + slot;
+    nrows = hbase < H ? min(16, qlen - t0) : 0;  // waves past the last head only help staging
+    pos0 = ctx - qlen + t0;
+  }
+  auto row_tok = [&](int r) -> size_t { return (size_t)(q0 + (DEC ? 0 : t0 + r)); };
+  auto row_head = [&](int r) -> int { return DEC ? hbase + r : hbase; };
+  auto row_pos = [&](int r) -> int { return DEC ? pos0 : pos0 + r; };
   unsigned* pm = PM + (size_t)wave * 16 * SS;
 
   bf16x8 qf[KW32];
-  f32x4 acc[R16];
+  f32x4 acc[NT];
   float mrow[4], lrow[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -262,13 +282,13 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
     lrow[i] = 0.f;
   }
 #pragma unroll
-  for (int vt = 0; vt < R16; ++vt) acc[vt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int vt = 0; vt < NT; ++vt) acc[vt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int ks = 0; ks < KW32; ++ks) {
     qf[ks] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-    if (own && r16 < nq) {
-      const size_t tok = (size_t)(q0 + t0 + r16);
-      const int d = 32 * ks + 8 * quad;
+    if (r16 < nrows) {
+      const size_t tok = row_tok(r16);
+      const int h = row_head(r16), d = 32 * ks + 8 * quad;
       if (d < R) {
         qf[ks] = ld8(q_lat + (tok * H + h) * R + d);
       } else {  // rotary part: entry e pairs with e +- P/2
@@ -276,7 +296,7 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
         const int e = d - R, pi = e < half ? e : e - half;
         const bf16_t* qr = q + (tok * H + h) * (size_t)(D + P) + D;
         const bf16x8 u = ld8(qr + pi), w = ld8(qr + half + pi);
-        const float* cs = table + (size_t)min(max(pos0 + r16, 0), n_pos - 1) * P;
+        const float* cs = table + (size_t)min(max(row_pos(r16), 0), n_pos - 1) * P;
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           const float c = cs[pi + k], sn = cs[half + pi + k], uu = bf2f(u[k]), ww = bf2f(w[k]);
@@ -285,11 +305,14 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
       }
     }
   }
-  const int j_hi = pos0 + nq;
+  // visible keys of the tile: [j_lo, j_hi); pages [p_lo, p_hi), this split's share of them
+  const int j_hi = DEC ? ctx : pos0 + min(16, qlen - t0);
   const int j_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
   const int p_lo = j_lo / PAGE, p_hi = (j_hi + PAGE - 1) / PAGE;
+  const int per = (p_hi - p_lo + nsplit - 1) / nsplit;
+  const int my_lo = p_lo + split * per, my_hi = min(p_hi, my_lo + per);
 
-  for (int pg = p_lo; pg < p_hi; ++pg) {
+  for (int pg = my_lo; pg < my_hi; ++pg) {
     const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
     const int jb = pg * PAGE;
     __syncthreads();  // the page before is consumed
@@ -305,7 +328,7 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
       }
     }
     __syncthreads();
-    if (own) {
+    if (nrows > 0) {
       f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KW32; ++ks) {
@@ -317,10 +340,10 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
       f32x4 cf;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int qi = 4 * quad + i;
-        const int d0 = pos0 + qi - (jb + r16), d1 = d0 - 16;
-        const bool ok0 = qi < nq && d0 >= 0 && (window <= 0 || d0 < window);
-        const bool ok1 = qi < nq && d1 >= 0 && (window <= 0 || d1 < window);
+        const int r = 4 * quad + i;
+        const int d0 = row_pos(r) - (jb + r16), d1 = d0 - 16;
+        const bool ok0 = r < nrows && d0 >= 0 && (window <= 0 || d0 < window);
+        const bool ok1 = r < nrows && d1 >= 0 && (window <= 0 || d1 < window);
         const float s0 = ok0 ? c0[i] * scale : -INFINITY, s1 = ok1 ? c1[i] * scale : -INFINITY;
         float mx = fmaxf(s0, s1);
 #pragma unroll
@@ -335,38 +358,49 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
         mrow[i] = m_new;
         const bf16_t h0 = f2bf(p0), h1 = f2bf(p1);
         const bf16_t l0 = f2bf(p0 - bf2f(h0)), l1 = f2bf(p1 - bf2f(h1));
-        pm[qi * SS + r16] = (unsigned)__builtin_bit_cast(unsigned short, h0) |
-                            ((unsigned)__builtin_bit_cast(unsigned short, l0) << 16);
-        pm[qi * SS + 16 + r16] = (unsigned)__builtin_bit_cast(unsigned short, h1) |
-                                 ((unsigned)__builtin_bit_cast(unsigned short, l1) << 16);
+        pm[r * SS + r16] = (unsigned)__builtin_bit_cast(unsigned short, h0) |
+                           ((unsigned)__builtin_bit_cast(unsigned short, l0) << 16);
+        pm[r * SS + 16 + r16] = (unsigned)__builtin_bit_cast(unsigned short, h1) |
+                                ((unsigned)__builtin_bit_cast(unsigned short, l1) << 16);
       }
 #pragma unroll
-      for (int vt = 0; vt < R16; ++vt) acc[vt] *= cf;
+      for (int vt = 0; vt < NT; ++vt) acc[vt] *= cf;
     }
     __syncthreads();  // the wave's weights are in its tile
-    if (own) {
+    if (nrows > 0) {
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(pm + r16 * SS + 16 * kb + 4 * quad);
 #pragma unroll
-        for (int vt = 0; vt < R16; ++vt) {
-          const bf16x4 v4 = *reinterpret_cast<const bf16x4*>(VT + (size_t)(16 * vt + r16) * VS + 16 * kb + 4 * quad);
+        for (int vt = 0; vt < NT; ++vt) {
+          const bf16x4 v4 = *reinterpret_cast<const bf16x4*>(VT + (size_t)(16 * (part * NT + vt) + r16) * VS + 16 * kb +
+                                                             4 * quad);
           const bf16x8 bb = {v4[0], v4[0], v4[1], v4[1], v4[2], v4[2], v4[3], v4[3]};
           acc[vt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bb, acc[vt], 0, 0, 0);
         }
       }
     }
   }
-  if (!own) return;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int qi = 4 * quad + i;
-    if (qi >= nq) continue;
-    const size_t tok = (size_t)(q0 + t0 + qi);
-    float f = lrow[i] > 0.f ? 1.f / lrow[i] : 0.f;
-    if (gate) f /= 1.f + expf(-bf2f(gate[tok * gate_stride + h]));
+    const int r = 4 * quad + i;
+    if (r >= nrows) continue;
+    const size_t tok = row_tok(r);
+    const int h = row_head(r);
+    if (!DEC || nsplit == 1) {
+      float f = lrow[i] > 0.f ? 1.f / lrow[i] : 0.f;
+      if (gate) f /= 1.f + expf(-bf2f(gate[tok * gate_stride + h]));
 #pragma unroll
-    for (int vt = 0; vt < R16; ++vt) out[(tok * H + h) * R + 16 * vt + r16] = f2bf(acc[vt][i] * f);
+      for (int vt = 0; vt < NT; ++vt) out[(tok * H + h) * R + 16 * (part * NT + vt) + r16] = f2bf(acc[vt][i] * f);
+    } else {
+      float* pa = part_acc + ((tok * nsplit + split) * H + h) * (size_t)R;
+#pragma unroll
+      for (int vt = 0; vt < NT; ++vt) pa[16 * (part * NT + vt) + r16] = acc[vt][i];
+      if (part == 0 && r16 == 0) {
+        part_ml[((tok * nsplit + split) * H + h) * 2] = mrow[i];
+        part_ml[((tok * nsplit + split) * H + h) * 2 + 1] = lrow[i];
+      }
+    }
   }
 }
 
@@ -381,20 +415,59 @@ bool mfma_usable(int R, int P, int D) {
          (R == 64 && (P == 64 || P == 32));
 }
 
-template <int KW32, int R16>
-int launch_mfma(dim3 grid, int nthr, size_t lds, hipStream_t st, const bf16_t* q, const bf16_t* q_lat,
-                const bf16_t* cache, const int* bt, int max_pages, const int* cu_q, const int* ctx_len,
-                const float* table, int n_pos, const bf16_t* gate, int64_t gate_stride, bf16_t* out, int H, int HG, int D,
-                float scale, int window) {
+struct MfmaArgs {
+  const bf16_t *q, *q_lat, *cache;
+  const int* bt;
+  int max_pages;
+  const int *cu_q, *ctx_len;
+  const float* table;
+  int n_pos;
+  const bf16_t* gate;
+  int64_t gate_stride;
+  bf16_t* out;
+  float *part_acc, *part_ml;
+  int H, D;
+  float scale;
+  int window, nsplit;
+};
+
+template <int KW32, int R16, int RS, bool DEC>
+int launch_mfma(dim3 grid, int nthr, int hg, hipStream_t st, const MfmaArgs& a) {
   static bool raised = false;  // once per kernel: no attribute call inside a stream capture later
   if (!raised) {
-    HIP_RET(hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<KW32, R16>,
+    HIP_RET(hipFuncSetAttribute((const void*)latent_attn_mfma_kernel<KW32, R16, RS, DEC>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     raised = true;
   }
-  hipLaunchKernelGGL((latent_attn_mfma_kernel<KW32, R16>), grid, dim3(nthr), lds, st, q, q_lat, cache, bt, max_pages,
-                     cu_q, ctx_len, table, n_pos, gate, gate_stride, out, H, HG, D, scale, window);
+  const size_t lds = mfma_lds_bytes(R16 * 16, KW32 * 32 - R16 * 16, nthr / 64);
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<KW32, R16, RS, DEC>), grid, dim3(nthr), lds, st, a.q, a.q_lat, a.cache,
+                     a.bt, a.max_pages, a.cu_q, a.ctx_len, a.table, a.n_pos, a.gate, a.gate_stride, a.out, a.part_acc,
+                     a.part_ml, a.H, hg, a.D, a.scale, a.window, a.nsplit);
   return (int)hipGetLastError();
+}
+
+// Prompt portions: RS waves per head (2 for the largest latent, so that the accumulators stay in registers), up to
+// 8 waves a workgroup. Decoding: 4 waves on the 16 heads of a head group.
+template <bool DEC>
+int dispatch_mfma(int R, int P, int B, int max_q, hipStream_t st, const MfmaArgs& a) {
+#define GO(KW32, R16, RS)                                                                      \
+  do {                                                                                         \
+    if (DEC) {                                                                                 \
+      const dim3 grid((a.H + 15) / 16, B, a.nsplit);                                           \
+      return launch_mfma<KW32, R16, 4, true>(grid, 256, 16, st, a);                            \
+    }                                                                                          \
+    const int hg = a.H < 8 / RS ? a.H : 8 / RS, n_groups = (a.H + hg - 1) / hg;                \
+    const dim3 grid(((max_q + 15) / 16) * n_groups, B, 1);                                     \
+    return launch_mfma<KW32, R16, RS, false>(grid, 64 * hg * RS, hg, st, a);                   \
+  } while (0)
+  if (R == 512) GO(18, 32, 2);
+  if (R == 256 && P == 64) GO(10, 16, 1);
+  if (R == 256) GO(9, 16, 1);
+  if (R == 128 && P == 64) GO(6, 8, 1);
+  if (R == 128) GO(5, 8, 1);
+  if (P == 64) GO(4, 4, 1);
+  GO(3, 4, 1);
+#undef GO
 }
 
 // Merge of the key-range splits of one (token, head): grid (T, H).
@@ -468,25 +541,23 @@ extern "C" int areal_latent_attn(const void* q, const void* q_lat, const void* c
                                  int nsplit, int dt, int matrix_cores, hipStream_t st) {
   if (B == 0 || T == 0) return 0;
   if (H < 1 || R < 1 || P % 2 || nsplit < 1 || n_pos < 1) return -1;
-  if (matrix_cores && dt == 0 && nsplit == 1 && max_q > 1 && mfma_usable(R, P, D)) {
-    const int hg = H < 8 ? H : 8, n_groups = (H + hg - 1) / hg;
-    const dim3 mgrid(((max_q + 15) / 16) * n_groups, B, 1);
-    const size_t mlds = mfma_lds_bytes(R, P, hg);
-#define MFMA_ARGS                                                                                                 \
-  mgrid, 64 * hg, mlds, st, (const bf16_t*)q, (const bf16_t*)q_lat, (const bf16_t*)cache, block_tables, max_pages, \
-      cu_q, ctx_len, table, n_pos, (const bf16_t*)gate, gate_stride, (bf16_t*)out, H, hg, D, scale, window
-    if (R == 512) return launch_mfma<18, 32>(MFMA_ARGS);
-    if (R == 256) return P == 64 ? launch_mfma<10, 16>(MFMA_ARGS) : launch_mfma<9, 16>(MFMA_ARGS);
-    if (R == 128) return P == 64 ? launch_mfma<6, 8>(MFMA_ARGS) : launch_mfma<5, 8>(MFMA_ARGS);
-    return P == 64 ? launch_mfma<4, 4>(MFMA_ARGS) : launch_mfma<3, 4>(MFMA_ARGS);
-#undef MFMA_ARGS
+  if (nsplit > 1 && (!part_acc || !part_ml)) return -3;
+  if (matrix_cores && dt == 0 && mfma_usable(R, P, D) && (max_q > 1 ? nsplit == 1 : true)) {
+    const MfmaArgs a{(const bf16_t*)q, (const bf16_t*)q_lat, (const bf16_t*)cache, block_tables, max_pages, cu_q,
+                     ctx_len, table, n_pos, (const bf16_t*)gate, gate_stride, (bf16_t*)out, part_acc, part_ml, H, D,
+                     scale, window, nsplit};
+    if (max_q > 1) return dispatch_mfma<false>(R, P, B, max_q, st, a);
+    const int e = dispatch_mfma<true>(R, P, B, 1, st, a);
+    if (e == 0 && nsplit > 1)
+      hipLaunchKernelGGL(latent_attn_combine_kernel<bf16_t>, dim3(T, H), dim3(128), 0, st, part_acc, part_ml,
+                         (const bf16_t*)gate, gate_stride, (bf16_t*)out, H, R, nsplit);
+    return e ? e : (int)hipGetLastError();
   }
   int want = 1;
   while (want < 8 && want < max_q) want <<= 1;
   LatentShape sh;
   if (!pick_shape(H, D, P, R, want, &sh)) return -2;
   const size_t lds = sh.floats() * sizeof(float);
-  if (nsplit > 1 && (!part_acc || !part_ml)) return -3;
   const int n_groups = (H + sh.HG - 1) / sh.HG;
   const dim3 grid(((max_q + sh.BQ - 1) / sh.BQ) * n_groups, B, nsplit);
 #define LAUNCH(TT)                                                                                                  \
