@@ -226,7 +226,7 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(
 //   decoding        (DEC = true):  the 16 heads of a head group of ONE query; grid z = splits of the key range.
 // RS waves share a tile's rows: each computes the scores (cheap beside p.c) and owns R / RS of the output columns,
 // which keeps the fp32 accumulators of large latents in registers. Per 32-key page:
-//   stage   the page's [c | r] rows -> LDS KT [32][KW + 8] (bf16), and the latent part transposed -> VT [R][32 + 8]
+//   stage   the page's [c | r] rows -> LDS KT [32][KW + 8] (bf16), and the latent part transposed -> VT [R][32 + 4]
 //   scores  rows (registers: absorbed query | rotated rotary part, bf16) x KT^T, bf16 MFMA 16x16x32 with fp32
 //           accumulation; scale and mask in fp32; running maximum / denominator of the 16 rows in registers (a row's
 //           keys sit in the 16 lanes of one quad); the weight p (fp32) goes into the wave's own LDS tile as the pair
@@ -241,7 +241,7 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
     const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, const bf16_t* __restrict__ gate,
     int64_t gate_stride, bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, int H,
     int HG, int D, float scale, int window, int nsplit) {
-  constexpr int KW = KW32 * 32, R = R16 * 16, P = KW - R, KS = KW + 8, VS = PAGE + 8, SS = PAGE + 4, NT = R16 / RS;
+  constexpr int KW = KW32 * 32, R = R16 * 16, P = KW - R, KS = KW + 8, VS = PAGE + 4, SS = PAGE + 4, NT = R16 / RS;
   static_assert(R16 % RS == 0, "output tiles split evenly over the waves of a row tile");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16_t* KT = reinterpret_cast<bf16_t*>(smem);                  // [32][KS]
@@ -322,12 +322,16 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
       bf16x8 x = ld8(kp + (size_t)key * KW + 8 * dv);
       if (jb + key >= j_hi) x = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};  // rows past the last key may hold anything
       st8(KT + (size_t)key * KS + 8 * dv, x);
-      if (8 * dv < R) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) VT[(size_t)(8 * dv + e) * VS + key] = x[e];
-      }
     }
     __syncthreads();
+    // the latent part once more, transposed, for p.c: consecutive lanes take consecutive KEYS, so that their 2-byte
+    // stores fall into neighbouring banks (walking the columns instead puts a whole wave on one bank)
+    for (int i = tid; i < PAGE * (R / 8); i += nthr) {
+      const int key = i % PAGE, dv = i / PAGE;
+      const bf16x8 x = ld8(KT + (size_t)key * KS + 8 * dv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) VT[(size_t)(8 * dv + e) * VS + key] = x[e];
+    }
     if (nrows > 0) {
       f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -405,7 +409,7 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
 }
 
 size_t mfma_lds_bytes(int R, int P, int waves) {
-  return (size_t)PAGE * (R + P + 8) * 2 + (size_t)R * (PAGE + 8) * 2 + (size_t)waves * 16 * (PAGE + 4) * 4;
+  return (size_t)PAGE * (R + P + 8) * 2 + (size_t)R * (PAGE + 4) * 2 + (size_t)waves * 16 * (PAGE + 4) * 4;
 }
 
 // Shapes the matrix-core kernel is instantiated for: (latent size, rotary size), unrotated key size D.

@@ -450,7 +450,8 @@ __global__ void __launch_bounds__(256) moe_combine_w32_kernel(const T* __restric
                                                               const float* __restrict__ w, T* __restrict__ out, int k,
                                                               int H) {
   const int64_t t = blockIdx.x;
-  for (int c = threadIdx.x; c < H; c += 256) {
+  const int c = blockIdx.y * 256 + threadIdx.x;  // one column per thread
+  if (c < H) {
     float a = 0.f;
     for (int j = 0; j < k; ++j) a += w[t * k + j] * mo_ld<T>(src, (size_t)inv[t * k + j] * H + c);
     mo_st<T>(out, (size_t)t * H + c, a);
@@ -477,10 +478,10 @@ extern "C" int areal_moe_combine_w32(const void* src, const int64_t* inv, const 
   if (T == 0) return 0;
   if (k < 1) return -3;
   if (dt == 0)
-    hipLaunchKernelGGL(moe_combine_w32_kernel<bf16_t>, dim3((unsigned)T), dim3(256), 0, st, (const bf16_t*)src, inv, w,
+    hipLaunchKernelGGL(moe_combine_w32_kernel<bf16_t>, dim3((unsigned)T, (H + 255) / 256), dim3(256), 0, st, (const bf16_t*)src, inv, w,
                        (bf16_t*)out, k, H);
   else
-    hipLaunchKernelGGL(moe_combine_w32_kernel<float>, dim3((unsigned)T), dim3(256), 0, st, (const float*)src, inv, w,
+    hipLaunchKernelGGL(moe_combine_w32_kernel<float>, dim3((unsigned)T, (H + 255) / 256), dim3(256), 0, st, (const float*)src, inv, w,
                        (float*)out, k, H);
   return (int)hipGetLastError();
 }

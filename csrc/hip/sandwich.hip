@@ -22,22 +22,25 @@ template <typename T> DEVINL void stf(T* p, size_t i, float v);
 template <> DEVINL void stf<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f2bf(v); }
 template <> DEVINL void stf<float>(float* p, size_t i, float v) { p[i] = v; }
 
-// Sum over the 256 threads of a workgroup; every thread gets the result. `red` holds 4 floats.
+// Sum over the threads of a workgroup (a multiple of 64, at most 1024); every thread gets the result. `red` holds 16
+// floats. Every thread adds the waves' sums in the same order, so all of them see the same bits.
 DEVINL float block_sum(float v, float* red) {
   v = wave_sum(v);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
   __syncthreads();
-  return red[0] + red[1] + red[2] + red[3];
+  float s = 0.f;
+  for (int w = 0; w < (int)(blockDim.x >> 6); ++w) s += red[w];
+  return s;
 }
 
 // (mean, 1 / sqrt(var + eps)) of the W floats in `row` (LDS); every thread gets both.
 DEVINL void row_stats(const float* row, int W, float eps, float* red, float& mean, float& rstd) {
   float s = 0.f;
-  for (int i = threadIdx.x; i < W; i += 256) s += row[i];
+  for (int i = threadIdx.x; i < W; i += blockDim.x) s += row[i];
   mean = block_sum(s, red) / (float)W;
   float v = 0.f;
-  for (int i = threadIdx.x; i < W; i += 256) {
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
     const float d = row[i] - mean;
     v += d * d;
   }
@@ -56,17 +59,17 @@ DEVINL int row_of(const int* __restrict__ cu_q, int B, int t) {
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256) layer_norm32_kernel(const float* __restrict__ x, const T* __restrict__ w,
+__global__ void __launch_bounds__(1024) layer_norm32_kernel(const float* __restrict__ x, const T* __restrict__ w,
                                                            const T* __restrict__ b, float* __restrict__ o32,
                                                            T* __restrict__ oc, int W, float eps) {
   extern __shared__ float row[];
   float* red = row + W;
   const size_t base = (size_t)blockIdx.x * W;
-  for (int i = threadIdx.x; i < W; i += 256) row[i] = x[base + i];
+  for (int i = threadIdx.x; i < W; i += blockDim.x) row[i] = x[base + i];
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
-  for (int i = threadIdx.x; i < W; i += 256) {
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
     const float h = (row[i] - mean) * rstd * ldf<T>(w, i) + ldf<T>(b, i);
     if (o32) o32[base + i] = h;
     if (oc) stf<T>(oc, base + i, h);
@@ -74,14 +77,14 @@ __global__ void __launch_bounds__(256) layer_norm32_kernel(const float* __restri
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256) gated_norm_add_kernel(
+__global__ void __launch_bounds__(1024) gated_norm_add_kernel(
     float* __restrict__ x, const T* __restrict__ y, const T* __restrict__ gate, const T* __restrict__ w,
     const T* __restrict__ b, const T* __restrict__ scale, const T* __restrict__ nw, const T* __restrict__ nb,
     float* __restrict__ h32, T* __restrict__ hc, int W, float eps) {
   extern __shared__ float row[];
   float* red = row + W;
   const size_t base = (size_t)blockIdx.x * W;
-  for (int i = threadIdx.x; i < W; i += 256) {
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float z = ldf<T>(y, base + i);
     if (gate) z /= 1.f + expf(-ldf<T>(gate, base + i));
     row[i] = z;
@@ -89,7 +92,7 @@ __global__ void __launch_bounds__(256) gated_norm_add_kernel(
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
-  for (int i = threadIdx.x; i < W; i += 256) {
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float r = (row[i] - mean) * rstd * ldf<T>(w, i) + ldf<T>(b, i);
     if (scale) r *= ldf<T>(scale, i);
     const float nx = x[base + i] + r;
@@ -99,7 +102,7 @@ __global__ void __launch_bounds__(256) gated_norm_add_kernel(
   if (!nw) return;
   __syncthreads();
   row_stats(row, W, eps, red, mean, rstd);
-  for (int i = threadIdx.x; i < W; i += 256) {
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
     const float h = (row[i] - mean) * rstd * ldf<T>(nw, i) + ldf<T>(nb, i);
     if (h32) h32[base + i] = h;
     if (hc) stf<T>(hc, base + i, h);
@@ -114,17 +117,17 @@ __global__ void __launch_bounds__(256) canon_conv_kernel(const float* __restrict
                                                          const int* __restrict__ first_pos,
                                                          const int* __restrict__ state_slots, T* __restrict__ out,
                                                          int B, int W, int taps) {
-  const int t = blockIdx.x, K = taps - 1;
+  const int t = blockIdx.x, K = taps - 1, c = blockIdx.y * 256 + threadIdx.x;  // one channel per thread
   const int b = row_of(cu_q, B, t);
   const int q0 = cu_q[b], n = cu_q[b + 1] - q0, off = t - q0;
   if (off >= n) return;  // a token no row owns
   const int slot = state_slots[b];
   if (slot < 0) {  // padding row: its values go nowhere, they only have to be finite
-    for (int c = threadIdx.x; c < W; c += 256) stf<T>(out, (size_t)t * W + c, h[(size_t)t * W + c]);
+    if (c < W) stf<T>(out, (size_t)t * W + c, h[(size_t)t * W + c]);
     return;
   }
   if (off >= K) {  // the whole history is inside the row
-    for (int c = threadIdx.x; c < W; c += 256) {
+    if (c < W) {
       float a = h[(size_t)t * W + c];
       for (int j = 0; j < taps; ++j) a += ldf<T>(w, (size_t)c * taps + j) * h[(size_t)(t - K + j) * W + c];
       stf<T>(out, (size_t)t * W + c, a);
@@ -140,7 +143,7 @@ __global__ void __launch_bounds__(256) canon_conv_kernel(const float* __restrict
     return p0 + p >= 0 ? sl[(size_t)(K + p) * W + c] : 0.f;
   };
   const int m = min(K, n);
-  for (int c = threadIdx.x; c < W; c += 256) {
+  if (c < W) {
     for (int i = 0; i < m; ++i) {
       float a = val(i, c);
       for (int j = 0; j < taps; ++j) a += ldf<T>(w, (size_t)c * taps + j) * val(i - K + j, c);
@@ -152,7 +155,7 @@ __global__ void __launch_bounds__(256) canon_conv_kernel(const float* __restrict
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256) embed_bigram_norm_kernel(
+__global__ void __launch_bounds__(1024) embed_bigram_norm_kernel(
     const int64_t* __restrict__ tokens, const T* __restrict__ embed, const T* __restrict__ bigram, int buckets,
     int64_t mul_prev, int64_t mul_cur, const T* __restrict__ w, const T* __restrict__ bias, float eps,
     const int* __restrict__ cu_q, const int* __restrict__ first_pos, const int* __restrict__ state_slots,
@@ -184,7 +187,7 @@ __global__ void __launch_bounds__(256) embed_bigram_norm_kernel(
   }
   __syncthreads();
   const int64_t r = big_row;
-  for (int i = threadIdx.x; i < W; i += 256) {
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
     float v = ldf<T>(embed, (size_t)tok * W + i);
     if (r >= 0) v += ldf<T>(bigram, (size_t)r * W + i);
     row[i] = v;
@@ -192,15 +195,19 @@ __global__ void __launch_bounds__(256) embed_bigram_norm_kernel(
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
-  for (int i = threadIdx.x; i < W; i += 256)
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
     out[(size_t)t * W + i] = (row[i] - mean) * rstd * ldf<T>(w, i) + ldf<T>(bias, i);
 }
 
 }  // namespace
 
+// Threads of a one-token workgroup: a few elements per thread, so that a launch of few tokens (a decode step) is not a
+// chain of dependent loads.
+static int row_threads(int W) { return W > 2048 ? 1024 : (W > 512 ? 512 : 256); }
+
 static int row_lds(int W, size_t* bytes) {
-  *bytes = (size_t)(W + 4) * sizeof(float);
-  return *bytes <= 64 * 1024 ? 0 : -2;  // rows up to 16380 channels
+  *bytes = (size_t)(W + 16) * sizeof(float);
+  return *bytes <= 64 * 1024 ? 0 : -2;  // rows up to 16368 channels
 }
 
 extern "C" int areal_layer_norm32(const float* x, const void* w, const void* b, float* o32, void* oc, int T, int W,
@@ -209,10 +216,10 @@ extern "C" int areal_layer_norm32(const float* x, const void* w, const void* b, 
   size_t lds;
   if (W <= 0 || row_lds(W, &lds)) return -2;
   if (dt == 0)
-    hipLaunchKernelGGL(layer_norm32_kernel<bf16_t>, dim3(T), dim3(256), lds, st, x, (const bf16_t*)w,
+    hipLaunchKernelGGL(layer_norm32_kernel<bf16_t>, dim3(T), dim3(row_threads(W)), lds, st, x, (const bf16_t*)w,
                        (const bf16_t*)b, o32, (bf16_t*)oc, W, eps);
   else
-    hipLaunchKernelGGL(layer_norm32_kernel<float>, dim3(T), dim3(256), lds, st, x, (const float*)w, (const float*)b,
+    hipLaunchKernelGGL(layer_norm32_kernel<float>, dim3(T), dim3(row_threads(W)), lds, st, x, (const float*)w, (const float*)b,
                        o32, (float*)nullptr, W, eps);
   return (int)hipGetLastError();
 }
@@ -224,11 +231,11 @@ extern "C" int areal_gated_norm_add(float* x, const void* y, const void* gate, c
   size_t lds;
   if (W <= 0 || row_lds(W, &lds)) return -2;
   if (dt == 0)
-    hipLaunchKernelGGL(gated_norm_add_kernel<bf16_t>, dim3(T), dim3(256), lds, st, x, (const bf16_t*)y,
+    hipLaunchKernelGGL(gated_norm_add_kernel<bf16_t>, dim3(T), dim3(row_threads(W)), lds, st, x, (const bf16_t*)y,
                        (const bf16_t*)gate, (const bf16_t*)w, (const bf16_t*)b, (const bf16_t*)scale,
                        (const bf16_t*)nw, (const bf16_t*)nb, h32, (bf16_t*)hc, W, eps);
   else
-    hipLaunchKernelGGL(gated_norm_add_kernel<float>, dim3(T), dim3(256), lds, st, x, (const float*)y,
+    hipLaunchKernelGGL(gated_norm_add_kernel<float>, dim3(T), dim3(row_threads(W)), lds, st, x, (const float*)y,
                        (const float*)gate, (const float*)w, (const float*)b, (const float*)scale, (const float*)nw,
                        (const float*)nb, h32, (float*)nullptr, W, eps);
   return (int)hipGetLastError();
@@ -238,12 +245,12 @@ extern "C" int areal_canon_conv(const float* h, const void* w, float* state, con
                                 const int* state_slots, void* out, int B, int T, int W, int taps, int dt,
                                 hipStream_t st) {
   if (T == 0 || B == 0) return 0;
-  if (taps < 1 || (taps > 1 && !state)) return -1;
+  if (taps < 1 || (taps > 1 && !state) || (W + 255) / 256 > 65535) return -1;
   if (dt == 0)
-    hipLaunchKernelGGL(canon_conv_kernel<bf16_t>, dim3(T), dim3(256), 0, st, h, (const bf16_t*)w, state, cu_q,
+    hipLaunchKernelGGL(canon_conv_kernel<bf16_t>, dim3(T, (W + 255) / 256), dim3(256), 0, st, h, (const bf16_t*)w, state, cu_q,
                        first_pos, state_slots, (bf16_t*)out, B, W, taps);
   else
-    hipLaunchKernelGGL(canon_conv_kernel<float>, dim3(T), dim3(256), 0, st, h, (const float*)w, state, cu_q,
+    hipLaunchKernelGGL(canon_conv_kernel<float>, dim3(T, (W + 255) / 256), dim3(256), 0, st, h, (const float*)w, state, cu_q,
                        first_pos, state_slots, (float*)out, B, W, taps);
   return (int)hipGetLastError();
 }
@@ -257,11 +264,11 @@ extern "C" int areal_embed_bigram_norm(const int64_t* tokens, const void* embed,
   if (W <= 0 || row_lds(W, &lds)) return -2;
   if (bigram && (buckets < 1 || !prev_state)) return -1;
   if (dt == 0)
-    hipLaunchKernelGGL(embed_bigram_norm_kernel<bf16_t>, dim3(T), dim3(256), lds, st, tokens, (const bf16_t*)embed,
+    hipLaunchKernelGGL(embed_bigram_norm_kernel<bf16_t>, dim3(T), dim3(row_threads(W)), lds, st, tokens, (const bf16_t*)embed,
                        (const bf16_t*)bigram, buckets, mul_prev, mul_cur, (const bf16_t*)w, (const bf16_t*)bias, eps,
                        cu_q, first_pos, state_slots, prev_state, out, B, W, vocab);
   else
-    hipLaunchKernelGGL(embed_bigram_norm_kernel<float>, dim3(T), dim3(256), lds, st, tokens, (const float*)embed,
+    hipLaunchKernelGGL(embed_bigram_norm_kernel<float>, dim3(T), dim3(row_threads(W)), lds, st, tokens, (const float*)embed,
                        (const float*)bigram, buckets, mul_prev, mul_cur, (const float*)w, (const float*)bias, eps,
                        cu_q, first_pos, state_slots, prev_state, out, B, W, vocab);
   return (int)hipGetLastError();
