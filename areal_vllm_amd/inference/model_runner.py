@@ -996,7 +996,7 @@ class HybridModelRunner(ModelRunner):
         if latent and self.device.type == "cuda":
             from ..ops import latent_attention as lattn
 
-            nsplit = max(lattn.decode_splits(Bp, m.window, self.max_context) for m in latent)
+            nsplit = max(lattn.decode_splits(Bp, m.window, self.max_context, m.H) for m in latent)
             if nsplit > 1:
                 ws = (torch.empty(Bp * nsplit * max(m.H * m.R for m in latent), dtype=torch.float32, device=self.device),
                       torch.empty(Bp * nsplit * max(m.H for m in latent) * 2, dtype=torch.float32, device=self.device))

@@ -19,12 +19,16 @@ CPU: PyTorch formulations of the same arithmetic (fp32).
 
 Cache layout: [pages, 32, R + P], token-major.
 """
+import os
 from typing import Optional, Tuple
 
 import torch
 
 from . import _lib as L
 from .attention import PAGE_SIZE
+
+
+DECODE_WORKGROUPS = int(os.environ.get("AREAL_LATENT_DECODE_WORKGROUPS", "256"))
 
 
 def alloc_latent_cache(num_pages: int, rank: int, rot: int, dtype, device) -> torch.Tensor:
@@ -81,11 +85,13 @@ def latent_prep(proj: torch.Tensor, q_rank: int, rank: int, rot: int, q_weight: 
     return cq
 
 
-def decode_splits(batch: int, window: int, max_context: int) -> int:
-    """Key-range splits of a decode launch: enough workgroups for the chip, down to one page each."""
+def decode_splits(batch: int, window: int, max_context: int, heads: int = 16) -> int:
+    """Key-range splits of a decode launch: about `DECODE_WORKGROUPS` workgroups (one per row, group of 16 heads and
+    split), down to one page each."""
     span = max_context if window <= 0 else min(window + PAGE_SIZE, max_context)
     pages = max(1, (span + PAGE_SIZE - 1) // PAGE_SIZE)
-    return int(max(1, min(512 // max(1, batch), pages, 32)))
+    groups = max(1, batch) * ((heads + 15) // 16)
+    return int(max(1, min(DECODE_WORKGROUPS // groups, pages, 32)))
 
 
 def latent_attention(q: torch.Tensor, q_lat: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,

@@ -235,13 +235,14 @@ __global__ void __launch_bounds__(256) latent_attn_kernel(
 //           carries 16 bits of p's mantissa (the latents themselves are bf16), fp32 accumulation in registers
 // KW32 = (R + P) / 32 k-steps of the scores, R16 = R / 16 output tiles.
 template <int KW32, int R16, int RS, bool DEC>
-__global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
+__global__ void __launch_bounds__(DEC ? 256 : 512) latent_attn_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ q_lat, const bf16_t* __restrict__ cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_len, const float* __restrict__ table, int n_pos, const bf16_t* __restrict__ gate,
     int64_t gate_stride, bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, int H,
     int HG, int D, float scale, int window, int nsplit) {
   constexpr int KW = KW32 * 32, R = R16 * 16, P = KW - R, KS = KW + 8, VS = PAGE + 4, SS = PAGE + 4, NT = R16 / RS;
+  constexpr int NB = (!DEC && KW32 >= 18) ? 3 : 4;  // the largest prompt instance has no registers to spare
   static_assert(R16 % RS == 0, "output tiles split evenly over the waves of a row tile");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16_t* KT = reinterpret_cast<bf16_t*>(smem);                  // [32][KS]
@@ -312,25 +313,71 @@ __global__ void __launch_bounds__(512) latent_attn_mfma_kernel(
   const int per = (p_hi - p_lo + nsplit - 1) / nsplit;
   const int my_lo = p_lo + split * per, my_hi = min(p_hi, my_lo + per);
 
+  // Decoding (256 threads): the NEXT page's rows are fetched into registers while this page is worked on, and its
+  // page number one step earlier still, so a workgroup's walk over its pages is not a chain of memory latencies.
+  constexpr int CH = PAGE * (KW / 8), NL = (CH + 255) / 256;
+  bf16x8 pre[DEC ? NL : 1];
+  int page_next = 0;
+  auto fetch = [&](int page) {
+    const bf16_t* kp = cache + (size_t)page * PAGE * KW;
+#pragma unroll
+    for (int u = 0; u < NL; ++u) {
+      const int i = tid + u * 256;
+      if (i < CH) pre[u] = ld8(kp + (size_t)(i / (KW / 8)) * KW + 8 * (i % (KW / 8)));
+    }
+  };
+  if (DEC && my_lo < my_hi) {
+    fetch(block_tables[(size_t)b * max_pages + my_lo]);
+    if (my_lo + 1 < my_hi) page_next = block_tables[(size_t)b * max_pages + my_lo + 1];
+  }
   for (int pg = my_lo; pg < my_hi; ++pg) {
-    const size_t page = (size_t)block_tables[(size_t)b * max_pages + pg];
     const int jb = pg * PAGE;
     __syncthreads();  // the page before is consumed
-    const bf16_t* kp = cache + page * PAGE * KW;
-    for (int i = tid; i < PAGE * (KW / 8); i += nthr) {
-      const int dv = i % (KW / 8), key = i / (KW / 8);
-      bf16x8 x = ld8(kp + (size_t)key * KW + 8 * dv);
-      if (jb + key >= j_hi) x = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};  // rows past the last key may hold anything
-      st8(KT + (size_t)key * KS + 8 * dv, x);
+    if (DEC) {
+#pragma unroll
+      for (int u = 0; u < NL; ++u) {
+        const int i = tid + u * 256;
+        if (i < CH) {
+          const int dv = i % (KW / 8), key = i / (KW / 8);
+          if (jb + key >= j_hi) pre[u] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};  // rows past the last key may hold anything
+          st8(KT + (size_t)key * KS + 8 * dv, pre[u]);
+        }
+      }
+      if (pg + 1 < my_hi) {
+        fetch(page_next);
+        if (pg + 2 < my_hi) page_next = block_tables[(size_t)b * max_pages + pg + 2];
+      }
+    } else {
+      const bf16_t* kp = cache + (size_t)block_tables[(size_t)b * max_pages + pg] * PAGE * KW;
+      // NB 16-byte loads of a thread are in flight before the first goes to LDS
+      for (int i0 = tid; i0 < CH; i0 += NB * nthr) {
+        bf16x8 x[NB];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+          const int i = i0 + u * nthr;
+          if (i < CH) x[u] = ld8(kp + (size_t)(i / (KW / 8)) * KW + 8 * (i % (KW / 8)));
+        }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+          const int i = i0 + u * nthr;
+          if (i < CH) {
+            const int dv = i % (KW / 8), key = i / (KW / 8);
+            if (jb + key >= j_hi) x[u] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};  // rows past the last key may hold anything
+            st8(KT + (size_t)key * KS + 8 * dv, x[u]);
+          }
+        }
+      }
     }
     __syncthreads();
-    // the latent part once more, transposed, for p.c: consecutive lanes take consecutive KEYS, so that their 2-byte
-    // stores fall into neighbouring banks (walking the columns instead puts a whole wave on one bank)
-    for (int i = tid; i < PAGE * (R / 8); i += nthr) {
-      const int key = i % PAGE, dv = i / PAGE;
-      const bf16x8 x = ld8(KT + (size_t)key * KS + 8 * dv);
+    // the latent part once more, transposed, for p.c: a thread takes two neighbouring keys and 8 columns and stores
+    // 4-byte key pairs; consecutive lanes take consecutive key pairs, so a wave's stores spread over the banks
+    // (walking the columns instead puts a whole wave on one bank)
+    for (int i = tid; i < (PAGE / 2) * (R / 8); i += nthr) {
+      const int kp2 = i % (PAGE / 2), dv = i / (PAGE / 2);
+      const bf16x8 x0 = ld8(KT + (size_t)(2 * kp2) * KS + 8 * dv), x1 = ld8(KT + (size_t)(2 * kp2 + 1) * KS + 8 * dv);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) VT[(size_t)(8 * dv + e) * VS + key] = x[e];
+      for (int e = 0; e < 8; ++e)
+        *reinterpret_cast<bf16x2*>(VT + (size_t)(8 * dv + e) * VS + 2 * kp2) = (bf16x2){x0[e], x1[e]};
     }
     if (nrows > 0) {
       f32x4 c0 = {0.f, 0.f, 0.f, 0.f}, c1 = {0.f, 0.f, 0.f, 0.f};
@@ -474,31 +521,35 @@ int dispatch_mfma(int R, int P, int B, int max_q, hipStream_t st, const MfmaArgs
 #undef GO
 }
 
-// Merge of the key-range splits of one (token, head): grid (T, H).
+// Merge of the key-range splits of one (token, head): grid (T, H). The splits' weights exp(m_s - m) (times gate / l)
+// are formed once in LDS; every thread then sums its columns over the splits with independent loads.
 template <typename T>
 __global__ void __launch_bounds__(128) latent_attn_combine_kernel(const float* __restrict__ part_acc,
                                                                   const float* __restrict__ part_ml,
                                                                   const T* __restrict__ gate, int64_t gate_stride,
                                                                   T* __restrict__ out, int H, int R, int nsplit) {
+  __shared__ float wsp[64];  // nsplit <= 64
   const size_t tok = blockIdx.x;
   const int h = blockIdx.y;
-  float m = -1e30f;
-  for (int s = 0; s < nsplit; ++s) m = fmaxf(m, part_ml[((tok * nsplit + s) * H + h) * 2]);
-  float l = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float* ml = part_ml + ((tok * nsplit + s) * H + h) * 2;
-    l += ml[1] * expf(ml[0] - m);
+  if (threadIdx.x < 64) {
+    const int s = threadIdx.x;
+    const float ms = s < nsplit ? part_ml[((tok * nsplit + s) * H + h) * 2] : -1e30f;
+    const float ls = s < nsplit ? part_ml[((tok * nsplit + s) * H + h) * 2 + 1] : 0.f;
+    const float m = wave_max(ms);
+    const float w = s < nsplit ? expf(ms - m) : 0.f;
+    const float l = wave_sum(ls * w);
+    float g = 1.f;
+    if (gate) g = 1.f / (1.f + expf(-ldf<T>(gate, tok * gate_stride + h)));
+    wsp[s] = l > 0.f ? w * g / l : 0.f;
   }
-  float g = 1.f;
-  if (gate) g = 1.f / (1.f + expf(-ldf<T>(gate, tok * gate_stride + h)));
-  const float inv = l > 0.f ? g / l : 0.f;
+  __syncthreads();
+  const float* base = part_acc + (tok * nsplit * H + h) * (size_t)R;
+  const size_t step = (size_t)H * R;
   for (int v = threadIdx.x; v < R; v += 128) {
     float a = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const float w = expf(part_ml[((tok * nsplit + s) * H + h) * 2] - m);
-      a += w * part_acc[((tok * nsplit + s) * H + h) * R + v];
-    }
-    stf<T>(out, (tok * H + h) * R + v, a * inv);
+#pragma unroll 4
+    for (int s = 0; s < nsplit; ++s) a += wsp[s] * base[s * step + v];
+    stf<T>(out, (tok * H + h) * R + v, a);
   }
 }
 
@@ -544,7 +595,7 @@ extern "C" int areal_latent_attn(const void* q, const void* q_lat, const void* c
                                  int B, int max_q, int T, int H, int D, int P, int R, float scale, int window,
                                  int nsplit, int dt, int matrix_cores, hipStream_t st) {
   if (B == 0 || T == 0) return 0;
-  if (H < 1 || R < 1 || P % 2 || nsplit < 1 || n_pos < 1) return -1;
+  if (H < 1 || R < 1 || P % 2 || nsplit < 1 || nsplit > 64 || n_pos < 1) return -1;
   if (nsplit > 1 && (!part_acc || !part_ml)) return -3;
   if (matrix_cores && dt == 0 && mfma_usable(R, P, D) && (max_q > 1 ? nsplit == 1 : true)) {
     const MfmaArgs a{(const bf16_t*)q, (const bf16_t*)q_lat, (const bf16_t*)cache, block_tables, max_pages, cu_q,
