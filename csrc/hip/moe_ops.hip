@@ -444,6 +444,26 @@ __global__ void __launch_bounds__(256) clamped_glu_kernel(const T* __restrict__ 
   }
 }
 
+// bf16 rows whose width is a multiple of 8: 16-byte loads and stores, 8 outputs a thread.
+__global__ void __launch_bounds__(256) clamped_glu_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
+                                                                 int64_t n, int F, float limit, float alpha) {
+  const int F8 = F / 8;
+  const int64_t total = n * (int64_t)F8;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t r = i / F8;
+    const int c = 8 * (int)(i - r * F8);
+    const bf16x8 g8 = ld8(gu + (size_t)r * 2 * F + c), u8 = ld8(gu + (size_t)r * 2 * F + F + c);
+    bf16x8 o;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float g = fminf(bf2f(g8[k]), limit);
+      const float u = fminf(fmaxf(bf2f(u8[k]), -limit), limit);
+      o[k] = f2bf(g / (1.f + expf(-alpha * g)) * (u + 1.f));
+    }
+    st8(out + (size_t)r * F + c, o);
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) moe_combine_w32_kernel(const T* __restrict__ src,
                                                               const int64_t* __restrict__ inv,
@@ -462,6 +482,13 @@ __global__ void __launch_bounds__(256) moe_combine_w32_kernel(const T* __restric
 extern "C" int areal_clamped_glu(const void* gu, void* out, int64_t n, int F, float limit, float alpha, int dt,
                                  hipStream_t st) {
   if (n == 0 || F == 0) return 0;
+  if (dt == 0 && F % 8 == 0 && (((uintptr_t)gu | (uintptr_t)out) & 15) == 0) {
+    const int64_t t8 = n * (int64_t)(F / 8);
+    const unsigned b8 = (unsigned)((t8 + 255) / 256 < 65535 * 16 ? (t8 + 255) / 256 : 65535 * 16);
+    hipLaunchKernelGGL(clamped_glu_bf16x8_kernel, dim3(b8), dim3(256), 0, st, (const bf16_t*)gu, (bf16_t*)out, n, F, limit,
+                       alpha);
+    return (int)hipGetLastError();
+  }
   const int64_t total = n * (int64_t)F;
   const unsigned blocks = (unsigned)((total + 255) / 256 < 65535 * 16 ? (total + 255) / 256 : 65535 * 16);
   if (dt == 0)

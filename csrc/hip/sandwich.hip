@@ -22,6 +22,19 @@ template <typename T> DEVINL void stf(T* p, size_t i, float v);
 template <> DEVINL void stf<bf16_t>(bf16_t* p, size_t i, float v) { p[i] = f2bf(v); }
 template <> DEVINL void stf<float>(float* p, size_t i, float v) { p[i] = v; }
 
+// Four consecutive elements at index i (a multiple of 4; the pointers are 16-byte aligned and rows are multiples of 4).
+template <typename T> DEVINL f32x4 ld4(const T* p, size_t i);
+template <> DEVINL f32x4 ld4<bf16_t>(const bf16_t* p, size_t i) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p + i);
+  return (f32x4){bf2f(v[0]), bf2f(v[1]), bf2f(v[2]), bf2f(v[3])};
+}
+template <> DEVINL f32x4 ld4<float>(const float* p, size_t i) { return *reinterpret_cast<const f32x4*>(p + i); }
+template <typename T> DEVINL void st4(T* p, size_t i, f32x4 v);
+template <> DEVINL void st4<bf16_t>(bf16_t* p, size_t i, f32x4 v) {
+  *reinterpret_cast<bf16x4*>(p + i) = (bf16x4){f2bf(v[0]), f2bf(v[1]), f2bf(v[2]), f2bf(v[3])};
+}
+template <> DEVINL void st4<float>(float* p, size_t i, f32x4 v) { *reinterpret_cast<f32x4*>(p + i) = v; }
+
 // Sum over the threads of a workgroup (a multiple of 64, at most 1024); every thread gets the result. `red` holds 16
 // floats. Every thread adds the waves' sums in the same order, so all of them see the same bits.
 DEVINL float block_sum(float v, float* red) {
@@ -58,54 +71,97 @@ DEVINL int row_of(const int* __restrict__ cu_q, int B, int t) {
   return lo;
 }
 
-template <typename T>
+template <typename T, bool V4>
 __global__ void __launch_bounds__(1024) layer_norm32_kernel(const float* __restrict__ x, const T* __restrict__ w,
-                                                           const T* __restrict__ b, float* __restrict__ o32,
-                                                           T* __restrict__ oc, int W, float eps) {
-  extern __shared__ float row[];
+                                                            const T* __restrict__ b, float* __restrict__ o32,
+                                                            T* __restrict__ oc, int W, float eps) {
+  extern __shared__ __attribute__((aligned(16))) float row[];
   float* red = row + W;
   const size_t base = (size_t)blockIdx.x * W;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) row[i] = x[base + i];
+  if (V4) {
+    for (int i = 4 * threadIdx.x; i < W; i += 4 * blockDim.x) *reinterpret_cast<f32x4*>(row + i) = ld4<float>(x, base + i);
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) row[i] = x[base + i];
+  }
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    const float h = (row[i] - mean) * rstd * ldf<T>(w, i) + ldf<T>(b, i);
-    if (o32) o32[base + i] = h;
-    if (oc) stf<T>(oc, base + i, h);
+  if (V4) {
+    for (int i = 4 * threadIdx.x; i < W; i += 4 * blockDim.x) {
+      const f32x4 h = (*reinterpret_cast<const f32x4*>(row + i) - mean) * rstd * ld4<T>(w, i) + ld4<T>(b, i);
+      if (o32) st4<float>(o32, base + i, h);
+      if (oc) st4<T>(oc, base + i, h);
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      const float h = (row[i] - mean) * rstd * ldf<T>(w, i) + ldf<T>(b, i);
+      if (o32) o32[base + i] = h;
+      if (oc) stf<T>(oc, base + i, h);
+    }
   }
 }
 
-template <typename T>
+// V4: rows that are multiples of 4 wide move as 16-byte (fp32) / 8-byte (bf16) vectors.
+template <typename T, bool V4>
 __global__ void __launch_bounds__(1024) gated_norm_add_kernel(
     float* __restrict__ x, const T* __restrict__ y, const T* __restrict__ gate, const T* __restrict__ w,
     const T* __restrict__ b, const T* __restrict__ scale, const T* __restrict__ nw, const T* __restrict__ nb,
     float* __restrict__ h32, T* __restrict__ hc, int W, float eps) {
-  extern __shared__ float row[];
+  extern __shared__ __attribute__((aligned(16))) float row[];
   float* red = row + W;
   const size_t base = (size_t)blockIdx.x * W;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float z = ldf<T>(y, base + i);
-    if (gate) z /= 1.f + expf(-ldf<T>(gate, base + i));
-    row[i] = z;
+  if (V4) {
+    for (int i = 4 * threadIdx.x; i < W; i += 4 * blockDim.x) {
+      f32x4 z = ld4<T>(y, base + i);
+      if (gate) {
+        const f32x4 g = ld4<T>(gate, base + i);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) z[k] /= 1.f + expf(-g[k]);
+      }
+      *reinterpret_cast<f32x4*>(row + i) = z;
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      float z = ldf<T>(y, base + i);
+      if (gate) z /= 1.f + expf(-ldf<T>(gate, base + i));
+      row[i] = z;
+    }
   }
   __syncthreads();
   float mean, rstd;
   row_stats(row, W, eps, red, mean, rstd);
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float r = (row[i] - mean) * rstd * ldf<T>(w, i) + ldf<T>(b, i);
-    if (scale) r *= ldf<T>(scale, i);
-    const float nx = x[base + i] + r;
-    x[base + i] = nx;
-    row[i] = nx;  // the element this thread owns in every pass
+  if (V4) {
+    for (int i = 4 * threadIdx.x; i < W; i += 4 * blockDim.x) {
+      f32x4 r = (*reinterpret_cast<const f32x4*>(row + i) - mean) * rstd * ld4<T>(w, i) + ld4<T>(b, i);
+      if (scale) r *= ld4<T>(scale, i);
+      const f32x4 nx = ld4<float>(x, base + i) + r;
+      st4<float>(x, base + i, nx);
+      *reinterpret_cast<f32x4*>(row + i) = nx;  // the elements this thread owns in every pass
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      float r = (row[i] - mean) * rstd * ldf<T>(w, i) + ldf<T>(b, i);
+      if (scale) r *= ldf<T>(scale, i);
+      const float nx = x[base + i] + r;
+      x[base + i] = nx;
+      row[i] = nx;  // the element this thread owns in every pass
+    }
   }
   if (!nw) return;
   __syncthreads();
   row_stats(row, W, eps, red, mean, rstd);
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    const float h = (row[i] - mean) * rstd * ldf<T>(nw, i) + ldf<T>(nb, i);
-    if (h32) h32[base + i] = h;
-    if (hc) stf<T>(hc, base + i, h);
+  if (V4) {
+    for (int i = 4 * threadIdx.x; i < W; i += 4 * blockDim.x) {
+      const f32x4 h = (*reinterpret_cast<const f32x4*>(row + i) - mean) * rstd * ld4<T>(nw, i) + ld4<T>(nb, i);
+      if (h32) st4<float>(h32, base + i, h);
+      if (hc) st4<T>(hc, base + i, h);
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      const float h = (row[i] - mean) * rstd * ldf<T>(nw, i) + ldf<T>(nb, i);
+      if (h32) h32[base + i] = h;
+      if (hc) stf<T>(hc, base + i, h);
+    }
   }
 }
 
@@ -210,17 +266,30 @@ static int row_lds(int W, size_t* bytes) {
   return *bytes <= 64 * 1024 ? 0 : -2;  // rows up to 16368 channels
 }
 
+// Threads of a one-token workgroup in the vector variants: four elements a thread and pass where the row allows.
+static int row_threads4(int W) {
+  const int t = ((W / 4 + 63) / 64) * 64;
+  return t > 1024 ? 1024 : (t < 64 ? 64 : t);
+}
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
 extern "C" int areal_layer_norm32(const float* x, const void* w, const void* b, float* o32, void* oc, int T, int W,
                                   float eps, int dt, hipStream_t st) {
   if (T == 0) return 0;
   size_t lds;
   if (W <= 0 || row_lds(W, &lds)) return -2;
-  if (dt == 0)
-    hipLaunchKernelGGL(layer_norm32_kernel<bf16_t>, dim3(T), dim3(row_threads(W)), lds, st, x, (const bf16_t*)w,
-                       (const bf16_t*)b, o32, (bf16_t*)oc, W, eps);
-  else
-    hipLaunchKernelGGL(layer_norm32_kernel<float>, dim3(T), dim3(row_threads(W)), lds, st, x, (const float*)w, (const float*)b,
-                       o32, (float*)nullptr, W, eps);
+  const bool v4 = W % 4 == 0 && aligned16(x) && aligned16(w) && aligned16(b) && aligned16(o32) && aligned16(oc);
+#define LN_LAUNCH(TT, V4, NTHR)                                                                               \
+  hipLaunchKernelGGL((layer_norm32_kernel<TT, V4>), dim3(T), dim3(NTHR), lds, st, x, (const TT*)w, (const TT*)b, \
+                     o32, (TT*)(dt == 0 ? oc : nullptr), W, eps)
+  if (dt == 0) {
+    if (v4) LN_LAUNCH(bf16_t, true, row_threads4(W));
+    else LN_LAUNCH(bf16_t, false, row_threads(W));
+  } else {
+    if (v4) LN_LAUNCH(float, true, row_threads4(W));
+    else LN_LAUNCH(float, false, row_threads(W));
+  }
+#undef LN_LAUNCH
   return (int)hipGetLastError();
 }
 
@@ -230,14 +299,20 @@ extern "C" int areal_gated_norm_add(float* x, const void* y, const void* gate, c
   if (T == 0) return 0;
   size_t lds;
   if (W <= 0 || row_lds(W, &lds)) return -2;
-  if (dt == 0)
-    hipLaunchKernelGGL(gated_norm_add_kernel<bf16_t>, dim3(T), dim3(row_threads(W)), lds, st, x, (const bf16_t*)y,
-                       (const bf16_t*)gate, (const bf16_t*)w, (const bf16_t*)b, (const bf16_t*)scale,
-                       (const bf16_t*)nw, (const bf16_t*)nb, h32, (bf16_t*)hc, W, eps);
-  else
-    hipLaunchKernelGGL(gated_norm_add_kernel<float>, dim3(T), dim3(row_threads(W)), lds, st, x, (const float*)y,
-                       (const float*)gate, (const float*)w, (const float*)b, (const float*)scale, (const float*)nw,
-                       (const float*)nb, h32, (float*)nullptr, W, eps);
+  const bool v4 = W % 4 == 0 && aligned16(x) && aligned16(y) && aligned16(gate) && aligned16(w) && aligned16(b) &&
+                  aligned16(scale) && aligned16(nw) && aligned16(nb) && aligned16(h32) && aligned16(hc);
+#define GN_LAUNCH(TT, V4, NTHR)                                                                                  \
+  hipLaunchKernelGGL((gated_norm_add_kernel<TT, V4>), dim3(T), dim3(NTHR), lds, st, x, (const TT*)y,             \
+                     (const TT*)gate, (const TT*)w, (const TT*)b, (const TT*)scale, (const TT*)nw, (const TT*)nb, \
+                     h32, (TT*)(dt == 0 ? hc : nullptr), W, eps)
+  if (dt == 0) {
+    if (v4) GN_LAUNCH(bf16_t, true, row_threads4(W));
+    else GN_LAUNCH(bf16_t, false, row_threads(W));
+  } else {
+    if (v4) GN_LAUNCH(float, true, row_threads4(W));
+    else GN_LAUNCH(float, false, row_threads(W));
+  }
+#undef GN_LAUNCH
   return (int)hipGetLastError();
 }
 
