@@ -55,7 +55,7 @@ def lufivik_dict(width, layers, heads, dim, rot, vdim, q_rank, kv_rank, window, 
              "mlp": {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": experts, "top": top}}}
     return {"architecture": "Lufivik", "layers": [json.loads(json.dumps(layer)) for _ in range(layers)],
             "norm": {"eps": 1e-5}, "canon": {"taps": 4},
-            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "vocab": VOCAB, "width": width}
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 36313, "mul_cur": 27191}}, "vocab": VOCAB, "width": width}
 
 
 def moe_twin_config(lcfg, width, layers, heads, experts, top):

@@ -272,7 +272,8 @@ __global__ void __launch_bounds__(DEC ? 256 : 512) latent_attn_mfma_kernel(
   auto row_tok = [&](int r) -> size_t { return (size_t)(q0 + (DEC ? 0 : t0 + r)); };
   auto row_head = [&](int r) -> int { return DEC ? hbase + r : hbase; };
   auto row_pos = [&](int r) -> int { return DEC ? pos0 : pos0 + r; };
-  unsigned* pm = PM + (size_t)wave * 16 * SS;
+  // decoding: the four waves of the tile compute the same weights; one tile holds them (written by the first wave)
+  unsigned* pm = PM + (size_t)(DEC ? 0 : wave) * 16 * SS;
 
   bf16x8 qf[KW32];
   f32x4 acc[NT];
@@ -407,12 +408,14 @@ __global__ void __launch_bounds__(DEC ? 256 : 512) latent_attn_mfma_kernel(
         cf[i] = __expf(mrow[i] - m_new);
         lrow[i] = lrow[i] * cf[i] + sum;
         mrow[i] = m_new;
-        const bf16_t h0 = f2bf(p0), h1 = f2bf(p1);
-        const bf16_t l0 = f2bf(p0 - bf2f(h0)), l1 = f2bf(p1 - bf2f(h1));
-        pm[r * SS + r16] = (unsigned)__builtin_bit_cast(unsigned short, h0) |
-                           ((unsigned)__builtin_bit_cast(unsigned short, l0) << 16);
-        pm[r * SS + 16 + r16] = (unsigned)__builtin_bit_cast(unsigned short, h1) |
-                                ((unsigned)__builtin_bit_cast(unsigned short, l1) << 16);
+        if (!DEC || part == 0) {
+          const bf16_t h0 = f2bf(p0), h1 = f2bf(p1);
+          const bf16_t l0 = f2bf(p0 - bf2f(h0)), l1 = f2bf(p1 - bf2f(h1));
+          pm[r * SS + r16] = (unsigned)__builtin_bit_cast(unsigned short, h0) |
+                             ((unsigned)__builtin_bit_cast(unsigned short, l0) << 16);
+          pm[r * SS + 16 + r16] = (unsigned)__builtin_bit_cast(unsigned short, h1) |
+                                  ((unsigned)__builtin_bit_cast(unsigned short, l1) << 16);
+        }
       }
 #pragma unroll
       for (int vt = 0; vt < NT; ++vt) acc[vt] *= cf;
@@ -490,7 +493,7 @@ int launch_mfma(dim3 grid, int nthr, int hg, hipStream_t st, const MfmaArgs& a) 
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     raised = true;
   }
-  const size_t lds = mfma_lds_bytes(R16 * 16, KW32 * 32 - R16 * 16, nthr / 64);
+  const size_t lds = mfma_lds_bytes(R16 * 16, KW32 * 32 - R16 * 16, DEC ? 1 : nthr / 64);
   hipLaunchKernelGGL((latent_attn_mfma_kernel<KW32, R16, RS, DEC>), grid, dim3(nthr), lds, st, a.q, a.q_lat, a.cache,
                      a.bt, a.max_pages, a.cu_q, a.ctx_len, a.table, a.n_pos, a.gate, a.gate_stride, a.out, a.part_acc,
                      a.part_ml, a.H, hg, a.D, a.scale, a.window, a.nsplit);
