@@ -323,8 +323,8 @@ class LatentAttentionMixer(nn.Module):
 
 
 class RoutedGLUExperts(nn.Module):
-    """Routed experts without biases: softmax over all router logits (fp32), the `top` largest scores are the
-    weights as they are; expert: down(g sigmoid(alpha g) (u + 1)) with g = min(gate h, limit), u = clamp(up h,
+    """Routed experts without biases: softmax over all router logits (an fp32 product on the fp32 normed input when
+    the caller has it), the `top` largest scores are the weights as they are; expert: down(g sigmoid(alpha g) (u + 1)) with g = min(gate h, limit), u = clamp(up h,
     -limit, limit). Tokens are sorted by expert and every expert runs on a contiguous slab (grouped kernels, row
     ranges on the device)."""
 
@@ -339,6 +339,8 @@ class RoutedGLUExperts(nn.Module):
     def forward(self, hc: torch.Tensor, h32: Optional[torch.Tensor]) -> torch.Tensor:
         if hc.dtype == torch.float32:
             z = F.linear(hc, self.router)
+        elif h32 is not None:  # the norm's fp32 output: the choice of experts does not see the bf16 rounding of h
+            z = F.linear(h32, self.router.float())
         elif hc.is_cuda:  # bf16 operands, fp32 accumulation AND fp32 logits
             z = torch.mm(hc, self.router.t(), out_dtype=torch.float32)
         else:
@@ -364,7 +366,8 @@ class SandwichBlock(nn.Module):
 
         mask = m.get("mask") or {}
         self.mix = LatentAttentionMixer(W, int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]),
-                                        int(m["q_rank"]), int(m["kv_rank"]), float(m["scale"]),
+                                        int(m["q_rank"]), int(m["kv_rank"]),
+                                        float(m.get("scale", (int(m["dim"]) + int(m["rot_dim"])) ** -0.5)),
                                         int(mask.get("size") or 0), float(m["rot"]["base"]), eps, dtype, device)
         self.norm1, self.norm1_bias, self.norm1b, self.norm1b_bias = vec(one=True), vec(), vec(one=True), vec()
         self.ls1 = vec(one=True)
@@ -399,7 +402,7 @@ class SandwichBlock(nn.Module):
         if self.mlp is None:
             return sandwich.gated_norm_add(x32, y, gate, self.norm1b, self.norm1b_bias, self.ls1, self.eps, next_norm)
         x32, h32, hc = sandwich.gated_norm_add(x32, y, gate, self.norm1b, self.norm1b_bias, self.ls1, self.eps,
-                                               (self.norm2, self.norm2_bias), want32=dtype == torch.float32)
+                                               (self.norm2, self.norm2_bias), want32=True)
         gate = F.linear(hc, self.rg2, self.rg2_bias)
         y = self.mlp(hc, h32)
         return sandwich.gated_norm_add(x32, y, gate, self.norm2b, self.norm2b_bias, self.ls2, self.eps, next_norm)

@@ -454,6 +454,9 @@ SHAPES = [
            width=40, vocab=67, eps=1e-3, taps=6, bigram=(7, 3, 2), loop=(0, 3, 2)),
     config([layer(4, 16, 8, 24, window=0)], width=24, bigram=None, taps=0),  # every earlier token seen; plain embedding
     config([layer(2, 8, 4, 8, ff=0), layer(2, 8, 4, 8, window=31)], width=56, taps=2, bigram=(1, 1, 1), loop=(1, 2, 3)),
+    # nothing a multiple of 4: width, ranks, head sizes, expert width, vocabulary
+    config([layer(3, 10, 6, 14, 18, 22, 13, ff=9, experts=4, top=2), layer(7, 6, 2, 5, 9, 11, 3, ff=0)], width=50, vocab=59,
+           taps=5, bigram=(97, 3, 11), loop=(0, 1, 3)),
     # sizes the matrix-core paths take
     config([layer(4, 64, 64, 64, 64, 128, 40, ff=64, experts=4, top=2), layer(8, 64, 32, 64, 128, 64, 70, ff=128)],
            width=64, loop=(0, 1, 2)),
