@@ -584,6 +584,53 @@ def test_served_from_a_checkpoint_directory(device, tmp_path):
         eng.destroy()
 
 
+def test_http_server_command_line_serves_a_checkpoint(tmp_path):
+    """The server's own command line -> engine -> POST /generate, greedy, against the float64 formulation."""
+    import asyncio
+    import socket
+    import threading
+
+    import requests
+    from aiohttp import web
+
+    from areal_vllm_amd.inference.server import InferenceServer, build_engine, parse_server_args
+    from areal_vllm_amd.models import build_model
+
+    cfg_dict = config([layer(2, 8, 4, 8, 12, 16, 11, ff=12, experts=3, top=2), layer(1, 8, 8, 16, 8, 8, 0, ff=0)], width=24,
+                      vocab=41, taps=2, loop=(0, 1, 2))
+    m = build_model(ModelConfig.from_hf_dict(cfg_dict), dtype=torch.float32)
+    m.flatten()
+    m.init_weights(seed=13)
+    m.save_checkpoint(str(tmp_path))
+    w = {k: v.float() for k, v in m.checkpoint_tensors().items()}
+    args, srv_cfg = parse_server_args(["--model-path", str(tmp_path), "--device", "cpu", "--num-pages", "16", "--dtype",
+                                       "float32", "--context-length", "128", "--max-running-requests", "2"])
+    eng = build_engine(args, srv_cfg)
+    with socket.socket() as sk:
+        sk.bind(("127.0.0.1", 0))
+        port = sk.getsockname()[1]
+    loop, started = asyncio.new_event_loop(), threading.Event()
+
+    def run():
+        asyncio.set_event_loop(loop)
+        runner = web.AppRunner(InferenceServer(eng).app)
+        loop.run_until_complete(runner.setup())
+        loop.run_until_complete(web.TCPSite(runner, "127.0.0.1", port).start())
+        started.set()
+        loop.run_forever()
+
+    threading.Thread(target=run, daemon=True).start()
+    assert started.wait(30)
+    try:
+        prompt = tokens_of(19, 41, 3)
+        r = requests.post(f"http://127.0.0.1:{port}/generate", json={
+            "input_ids": prompt, "sampling_params": {"max_new_tokens": 6, "temperature": 0.0}}, timeout=120).json()
+        assert r["output_ids"] == O.greedy(prompt, 6, w, cfg_dict)
+    finally:
+        loop.call_soon_threadsafe(loop.stop)
+        eng.destroy()
+
+
 def test_config_reader_and_checkpoint_save_then_load(tmp_path):
     cfg = ModelConfig.from_hf_dict(SHAPES[1])
     assert cfg.family == "lufivik" and cfg.n_layers == 3 and cfg.has_recurrent_state
